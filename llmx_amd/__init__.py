@@ -6,7 +6,7 @@ function over mixed batches, a scheduler, sampling, and hand-written gfx950 kern
 Importing the package touches neither the GPU nor the kernel library; both are needed from the first `Engine` on.
 """
 
-from .config import ConfigError, MiniMaxM3Config
+from .config import ConfigError, MiniMaxM3Config, NenotarConfig
 from .weights import RandomInit, WeightsError
 
 __version__ = "0.1.0"
@@ -32,5 +32,5 @@ def __getattr__(name):
     raise AttributeError(f"module 'llmx_amd' has no attribute {name!r}")
 
 
-__all__ = ["ConfigError", "MiniMaxM3Config", "RandomInit", "WeightsError", "Engine", "StepEntry", "StepError", "generate",
+__all__ = ["ConfigError", "MiniMaxM3Config", "NenotarConfig", "RandomInit", "WeightsError", "Engine", "StepEntry", "StepError", "generate",
            "Generator", "SamplingParams", "Scheduler", "Request", "write_random_model"]

@@ -2,5 +2,6 @@
 
 from .reader import ConfigError, KeyReader, read_json
 from .minimax_m3 import MiniMaxM3Config
+from .nenotar import NenotarConfig
 
-__all__ = ["ConfigError", "KeyReader", "read_json", "MiniMaxM3Config"]
+__all__ = ["ConfigError", "KeyReader", "read_json", "MiniMaxM3Config", "NenotarConfig"]

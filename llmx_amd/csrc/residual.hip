@@ -1,0 +1,140 @@
+// Kernels around the residual stream of layers whose mixer and feed-forward read the same rows: one norm pass with two
+// gains, the scaled join of both results, a normed join, and activations applied between two products.
+// Everything here is float32 arithmetic on float32 rows; only what a product reads next is stored in the activation type.
+#include "common.h"
+
+// ---------------------------------------------------------------------------
+// Two RMS norms of the same row with the same eps and different gains: r is formed once (the sum of squares in the
+// order of rmsnorm_kernel, so each output has the bits that kernel gives with its gain), out1 = x * (r * w1),
+// out2 = x * (r * w2).  out2 / w2 may be null.
+#define PAIR_THREADS 1024
+template <typename TO>
+__global__ void __launch_bounds__(PAIR_THREADS) rmsnorm_pair_kernel(const float* __restrict__ x, const float* __restrict__ w1,
+                                                                  const float* __restrict__ w2, float eps, TO* __restrict__ out1,
+                                                                  TO* __restrict__ out2, int n) {
+    __shared__ float scratch[PAIR_THREADS / 64];
+    const int r = blockIdx.x;
+    const float* row = x + (size_t)r * n;
+    const float s = block_sum<PAIR_THREADS / 64>(strided_squares<PAIR_THREADS>(row, n), scratch);
+    const float scale = 1.0f / sqrtf(s / (float)n + eps);
+    for (int i = threadIdx.x; i < n; i += PAIR_THREADS) {
+        const float v = row[i];
+        st(out1 + (size_t)r * n + i, v * (scale * w1[i]));
+        if (out2) st(out2 + (size_t)r * n + i, v * (scale * w2[i]));
+    }
+}
+
+extern "C" int llmx_rmsnorm_pair(const float* x, const float* w1, const float* w2, float eps, void* out1, void* out2, int out_dtype,
+                                 int rows, int n, hipStream_t stream) {
+    if (rows <= 0) return 0;
+    if (!w1 || !out1 || ((out2 != nullptr) != (w2 != nullptr))) return -2;
+    llmx_note_launch(LK_RMSNORM_PAIR);
+    if (out_dtype == LLMX_F32)
+        hipLaunchKernelGGL(rmsnorm_pair_kernel<float>, dim3(rows), dim3(PAIR_THREADS), 0, stream, x, w1, w2, eps, (float*)out1, (float*)out2, n);
+    else
+        hipLaunchKernelGGL(rmsnorm_pair_kernel<bf16_t>, dim3(rows), dim3(PAIR_THREADS), 0, stream, x, w1, w2, eps, (bf16_t*)out1, (bf16_t*)out2, n);
+    return LLMX_CHECK_LAUNCH();
+}
+
+// ---------------------------------------------------------------------------
+// x[t,i] += s1[i] * y1[t,i] + s2[i] * y2[t,i] (the second term only when y2 is given; a null scale is 1), and
+// optionally a copy of the new row in the activation type for the product that reads it next.
+template <typename TO>
+__global__ void __launch_bounds__(256) scale_add_kernel(float* __restrict__ x, const float* __restrict__ y1, const float* __restrict__ s1,
+                                                      const float* __restrict__ y2, const float* __restrict__ s2, TO* __restrict__ copy,
+                                                      int n, size_t total) {
+    const size_t at = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (at >= total) return;
+    const int i = (int)(at % (size_t)n);
+    float joined = y1[at] * (s1 ? s1[i] : 1.0f);
+    if (y2) joined = joined + y2[at] * (s2 ? s2[i] : 1.0f);
+    const float v = x[at] + joined;
+    x[at] = v;
+    if (copy) st(copy + at, v);
+}
+
+extern "C" int llmx_scale_add(float* x, const float* y1, const float* s1, const float* y2, const float* s2, void* copy, int copy_dtype,
+                              int rows, int n, hipStream_t stream) {
+    if (rows <= 0 || n <= 0) return 0;
+    llmx_note_launch(LK_SCALE_ADD);
+    const size_t total = (size_t)rows * n;
+    const dim3 grid((unsigned)((total + 255) / 256));
+    if (copy_dtype == LLMX_F32)
+        hipLaunchKernelGGL(scale_add_kernel<float>, grid, dim3(256), 0, stream, x, y1, s1, y2, s2, (float*)copy, n, total);
+    else
+        hipLaunchKernelGGL(scale_add_kernel<bf16_t>, grid, dim3(256), 0, stream, x, y1, s1, y2, s2, (bf16_t*)copy, n, total);
+    return LLMX_CHECK_LAUNCH();
+}
+
+// ---------------------------------------------------------------------------
+// x[t,:] += y[t,:] * (r * w[:]), r = 1 / sqrt(mean(y[t,:]^2) + eps): a result joined after its own RMS norm.
+__global__ void __launch_bounds__(256) rmsnorm_add_kernel(float* __restrict__ x, const float* __restrict__ y, const float* __restrict__ w,
+                                                        float eps, int n) {
+    __shared__ float scratch[4];
+    const int r = blockIdx.x;
+    const float* row = y + (size_t)r * n;
+    const float s = block_sum<4>(strided_squares<256>(row, n), scratch);
+    const float scale = 1.0f / sqrtf(s / (float)n + eps);
+    float* out = x + (size_t)r * n;
+    for (int i = threadIdx.x; i < n; i += 256) out[i] = out[i] + row[i] * (scale * w[i]);
+}
+
+extern "C" int llmx_rmsnorm_add(float* x, const float* y, const float* w, float eps, int rows, int n, hipStream_t stream) {
+    if (rows <= 0) return 0;
+    llmx_note_launch(LK_RMSNORM_ADD);
+    hipLaunchKernelGGL(rmsnorm_add_kernel, dim3(rows), dim3(256), 0, stream, x, y, w, eps, n);
+    return LLMX_CHECK_LAUNCH();
+}
+
+// ---------------------------------------------------------------------------
+// Activations between two products, float32 in, the activation type out.
+__device__ __forceinline__ float softplus_f(float v) { return log1pf(expf(-fabsf(v))) + fmaxf(v, 0.0f); }
+
+// xIELU with the two numbers (p, q) of `pq`: z > 0: softplus(p) z^2 + z/2; z <= 0: (1/2 + softplus(q)) (e^z - 1 - z) + z/2.
+template <typename TO>
+__global__ void __launch_bounds__(256) xielu_kernel(const float* __restrict__ z, const float* __restrict__ pq, TO* __restrict__ out, size_t total) {
+    const size_t at = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (at >= total) return;
+    const float up = softplus_f(pq[0]), down = 0.5f + softplus_f(pq[1]);
+    const float v = z[at];
+    const float y = v > 0.0f ? up * v * v + 0.5f * v : down * (expm1f(v) - v) + 0.5f * v;
+    st(out + at, y);
+}
+
+extern "C" int llmx_act_xielu(const float* z, const float* pq, void* out, int out_dtype, long total, hipStream_t stream) {
+    if (total <= 0) return 0;
+    llmx_note_launch(LK_ACT_XIELU);
+    const dim3 grid((unsigned)((total + 255) / 256));
+    if (out_dtype == LLMX_F32) hipLaunchKernelGGL(xielu_kernel<float>, grid, dim3(256), 0, stream, z, pq, (float*)out, (size_t)total);
+    else hipLaunchKernelGGL(xielu_kernel<bf16_t>, grid, dim3(256), 0, stream, z, pq, (bf16_t*)out, (size_t)total);
+    return LLMX_CHECK_LAUNCH();
+}
+
+// out[t,j] = gelu_tanh(z[t,j]) * table[ids[t], col0 + j], j < n: a gate on a slice of a token table's row.
+// gelu_tanh(v) = v/2 (1 + tanh(sqrt(2/pi) (v + 0.044715 v^3))).
+template <typename TT, typename TO>
+__global__ void __launch_bounds__(256) gelu_gather_kernel(const float* __restrict__ z, const TT* __restrict__ table, const int* __restrict__ ids,
+                                                        TO* __restrict__ out, int n, int col0, int table_ld, size_t total) {
+    const size_t at = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (at >= total) return;
+    const int t = (int)(at / (size_t)n), j = (int)(at % (size_t)n);
+    const float v = z[at];
+    const float g = 0.5f * v * (1.0f + tanhf(0.7978845608028654f * (v + 0.044715f * v * v * v)));
+    st(out + at, g * ld(table + (size_t)ids[t] * table_ld + col0 + j));
+}
+
+extern "C" int llmx_act_gelu_gather(const float* z, const void* table, int table_dtype, const int* ids, void* out, int out_dtype, int rows,
+                                    int n, int col0, int table_ld, hipStream_t stream) {
+    if (rows <= 0 || n <= 0) return 0;
+    if (col0 < 0 || col0 + n > table_ld) return -2;
+    llmx_note_launch(LK_ACT_GELU_GATHER);
+    const size_t total = (size_t)rows * n;
+    const dim3 grid((unsigned)((total + 255) / 256));
+#define LLMX_GG(TT, TO) hipLaunchKernelGGL((gelu_gather_kernel<TT, TO>), grid, dim3(256), 0, stream, z, (const TT*)table, ids, (TO*)out, n, col0, table_ld, total)
+    if (table_dtype == LLMX_F32 && out_dtype == LLMX_F32) LLMX_GG(float, float);
+    else if (table_dtype == LLMX_F32) LLMX_GG(float, bf16_t);
+    else if (out_dtype == LLMX_F32) LLMX_GG(bf16_t, float);
+    else LLMX_GG(bf16_t, bf16_t);
+#undef LLMX_GG
+    return LLMX_CHECK_LAUNCH();
+}

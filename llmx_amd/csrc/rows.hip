@@ -2,22 +2,23 @@
 #include "common.h"
 
 // ---------------------------------------------------------------------------
-// Embedding: x[t,:] = f32(table[id[t],:]).  Ids are checked on the host before any launch.
+// Embedding: x[t,:] = f32(table[id[t],:]) * scale (1 for a plain table).  Ids are checked on the host before any launch.
 template <typename TW>
-__global__ void embed_gather_kernel(const TW* __restrict__ table, const int* __restrict__ ids, float* __restrict__ x, int width) {
+__global__ void embed_gather_kernel(const TW* __restrict__ table, const int* __restrict__ ids, float* __restrict__ x, int width, float scale) {
     const int t = blockIdx.x;
     const TW* row = table + (size_t)ids[t] * width;
     float* out = x + (size_t)t * width;
-    for (int i = threadIdx.x; i < width; i += blockDim.x) out[i] = ld(row + i);
+    for (int i = threadIdx.x; i < width; i += blockDim.x) out[i] = ld(row + i) * scale;
 }
 
-extern "C" int llmx_embed_gather(const void* table, int table_dtype, const int* ids, float* x, int rows, int width, hipStream_t stream) {
+extern "C" int llmx_embed_gather(const void* table, int table_dtype, const int* ids, float* x, int rows, int width, float scale,
+                                 hipStream_t stream) {
     if (rows <= 0) return 0;
     llmx_note_launch(LK_EMBED_GATHER);
     if (table_dtype == LLMX_F32)
-        hipLaunchKernelGGL(embed_gather_kernel<float>, dim3(rows), dim3(256), 0, stream, (const float*)table, ids, x, width);
+        hipLaunchKernelGGL(embed_gather_kernel<float>, dim3(rows), dim3(256), 0, stream, (const float*)table, ids, x, width, scale);
     else
-        hipLaunchKernelGGL(embed_gather_kernel<bf16_t>, dim3(rows), dim3(256), 0, stream, (const bf16_t*)table, ids, x, width);
+        hipLaunchKernelGGL(embed_gather_kernel<bf16_t>, dim3(rows), dim3(256), 0, stream, (const bf16_t*)table, ids, x, width, scale);
     return LLMX_CHECK_LAUNCH();
 }
 

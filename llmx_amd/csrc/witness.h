@@ -48,7 +48,19 @@
     X(SAMPLE_TOPK, "sample_topk")                                                                                         \
     X(SAMPLE_RANKED, "sample_ranked")                                                                                     \
     X(SAMPLE_RANKED_SLICES, "sample_ranked.slices")                                                                       \
-    X(PENALIZE, "penalize")
+    X(PENALIZE, "penalize")                                                                                               \
+    X(RMSNORM_PAIR, "rmsnorm_pair")                                                                                       \
+    X(RMSNORM_ADD, "rmsnorm_add")                                                                                         \
+    X(SCALE_ADD, "scale_add")                                                                                             \
+    X(ACT_XIELU, "act.xielu")                                                                                             \
+    X(ACT_GELU_GATHER, "act.gelu_gather")                                                                                 \
+    X(GATED_SCAN, "gated_scan")                                                                                           \
+    X(GATED_SCAN_CHUNKS, "gated_scan.chunks")                                                                             \
+    X(LATENT_PREP, "latent_prep")                                                                                         \
+    X(LATENT_ATTENTION_GENERIC, "latent_attention.generic")                                                               \
+    X(LATENT_ATTENTION_MFMA, "latent_attention.mfma")                                                                     \
+    X(LATENT_ATTENTION_MERGE, "latent_attention.merge")                                                                   \
+    X(HEAD_GATE, "head_gate")
 
 enum LlmxLaunchKind : int {
 #define LLMX_X(id, name) LK_##id,

@@ -30,6 +30,7 @@ class EntryView:
     row0: int      # its first row in the step
     n: int         # its number of rows
     past: int      # tokens it held before the step
+    held: int = -1  # the slot that holds its state as the step found it, when the step writes another (`slot`); -1: the same
 
 
 class StepError(ValueError):
@@ -105,6 +106,7 @@ class StepState:
         self.rows = 0
         self.entries: List[EntryView] = []
         self.token_ids = self.positions = self.row_entry = self.entry_slots = self.pick = None
+        self.entry_held_slots = self.entry_rows = None
         self._tables: List[torch.Tensor] = []
         self.max_rows_per_entry = 0
         self._shared: Dict = {}

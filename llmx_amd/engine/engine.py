@@ -181,6 +181,11 @@ class Engine:
                 self._state.append(torch.zeros((self.cache.slots.capacity, *need.shape), dtype=getattr(torch, need.dtype), device=self.device))
             else:
                 self._state.append(None)
+        # which states a step must copy into its slot beforehand: those of mixers that step in place
+        writers = {e.cache: self.model.blocks[e.layer].mixer for e in self.spec.run_order if e.writes}
+        self._state_copied = [isinstance(need, StateNeed) and not getattr(writers[i], "steps_between_slots", False)
+                              for i, need in enumerate(needs)]
+        self._copy_state = any(self._state_copied)
         self._layer_caches: List[LayerCache] = []
         for e in self.spec.run_order:
             g = self._group_of[e.cache]
@@ -263,16 +268,17 @@ class Engine:
         return logits
 
     def _enter_shadow_slots(self, views: List[EntryView]) -> List[EntryView]:
-        """Each entry's state is copied into the slot its step writes, and the entry is pointed there; the slot it had
-        is not touched until the step commits."""
+        """Each entry is pointed at the slot its step writes; the slot it had (`held`) is not touched until the step
+        commits.  A mixer that reads the state from the held slot and writes the step's slot (`steps_between_slots`)
+        needs nothing more; for any other the state is copied into the step's slot first."""
         moved = []
         for v in views:
             to = self.cache.step_slot(v.request)
-            if to != v.slot:
-                for s in self._state:
-                    if s is not None:
+            if to != v.slot and self._copy_state:
+                for s, copies in zip(self._state, self._state_copied):
+                    if s is not None and copies:
                         s[to].copy_(s[v.slot])
-            moved.append(replace(v, slot=to))
+            moved.append(replace(v, slot=to, held=v.slot))
         return moved
 
     # -- wrappers over step, for one request (the reference's Model::prefill / step / score, runtime.hpp:1278-1385) --
@@ -329,7 +335,9 @@ class Engine:
             row_entry[v.row0:v.row0 + v.n] = i
             pick.extend(v.row0 + int(w) for w in e.want)
         slots = np.asarray([v.slot for v in views], dtype=np.int32)
-        arrays = [token_ids, positions, row_entry, slots, np.asarray(pick if pick else [0], dtype=np.int32)]
+        held = np.asarray([v.slot if v.held < 0 else v.held for v in views], dtype=np.int32)
+        entry_rows = np.asarray([[v.row0, v.n] for v in views], dtype=np.int32)
+        arrays = [token_ids, positions, row_entry, slots, np.asarray(pick if pick else [0], dtype=np.int32), held, entry_rows]
         for g in range(len(self.cache.groups)):
             tables = [self.cache.table(e.request, g) for e in entries]
             width = max(1, max(len(t) for t in tables))
@@ -345,7 +353,8 @@ class Engine:
         step.entries = views
         step.token_ids, step.positions, step.row_entry, step.entry_slots = dev[0], dev[1], dev[2], dev[3]
         step.pick = dev[4][:len(pick)]
-        step._tables = dev[5:]
+        step.entry_held_slots, step.entry_rows = dev[5], dev[6]
+        step._tables = dev[7:]
         step.max_rows_per_entry = max(v.n for v in views)
         step.observer = self.observer
 
@@ -355,7 +364,7 @@ class Engine:
         # scratch storage moves.  The row plan is copied to the device before the replay, outside the graph; the graph holds kernels only.
         key = None
         if self.graphs and self.observer is None and len(pick) > 0 and all(v.n == 1 for v in views):
-            key = (T, tuple(pick), tuple(a.shape for a in arrays[5:]), tuple(p.graph_key(step) for p in self._keyed_parts))
+            key = (T, tuple(pick), tuple(a.shape for a in arrays[7:]), tuple(p.graph_key(step) for p in self._keyed_parts))
             graph = self._graphs.get(key)
             if graph is not None and not graph.stale(self):
                 graph.graph.replay()
@@ -386,6 +395,8 @@ class Engine:
         for i, (entry, cache) in enumerate(zip(self.spec.run_order, self._layer_caches)):
             step.run_index = i
             self.model.blocks[entry.layer].forward(step, x, cache)
+            if step.observer is not None:
+                step.observe("layer", run_index=i, residual=x)
         W = step.pick.shape[0]
         if W == 0:
             return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=self.device)

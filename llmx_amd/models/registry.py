@@ -1,4 +1,4 @@
-"""One registry from an architecture's name (config.json `architectures[0]`) to its typed configuration and its model.
+"""One registry from an architecture's name (config.json `architectures[0]`, or `architecture`) to its typed configuration and its model.
 
 An entry holds the configuration class (`from_json(dict)`, `to_json()`) and the function that turns a configuration
 into a `ModelSpec`.  The lookup follows /root/reference/src/model/arch/registry.hpp:25-60: an unknown name is refused
@@ -46,7 +46,11 @@ def architectures() -> list[str]:
 
 
 def read_config(values: dict):
-    """The typed configuration of a parsed config.json, its class chosen by `architectures`."""
+    """The typed configuration of a parsed config.json, its class chosen by `architectures` (a list of one name) or,
+    for designs that spell it so, `architecture` (the name)."""
+    one = values.get("architecture") if isinstance(values, dict) else None
+    if isinstance(one, str) and "architectures" not in values:
+        return architecture_of(one).config_class.from_json(values)
     archs = values.get("architectures") if isinstance(values, dict) else None
     if not isinstance(archs, list) or len(archs) != 1 or not isinstance(archs[0], str):
         raise ConfigError("config: missing key architectures" if not archs else f"config: unsupported value for architectures ({archs!r})")

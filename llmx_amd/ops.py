@@ -53,7 +53,16 @@ def library_path() -> str:
 def _declare(h) -> None:
     P, I, F, L = c_void_p, c_int, c_float, c_long
     sigs = {
-        "llmx_embed_gather": [P, I, P, P, I, I, P],
+        "llmx_embed_gather": [P, I, P, P, I, I, F, P],
+        "llmx_rmsnorm_pair": [P, P, P, F, P, P, I, I, I, P],
+        "llmx_scale_add": [P, P, P, P, P, P, I, I, I, P],
+        "llmx_rmsnorm_add": [P, P, P, F, I, I, P],
+        "llmx_act_xielu": [P, P, P, I, L, P],
+        "llmx_act_gelu_gather": [P, P, I, P, P, I, I, I, I, I, P],
+        "llmx_mingru_scan": [P, P, P, P, P, P, P, P, I, I, I, P],
+        "llmx_latent_prep": [P, P, P, P, P, P, P, P, P, I, F, I, I, I, I, I, I, I, I, I, I, P],
+        "llmx_latent_attention_generic": [P, P, P, P, P, P, P, I, F, I, I, I, I, I, I, I, P],
+        "llmx_head_gate": [P, P, I, P, I, I, I, I, P],
         "llmx_rmsnorm": [P, P, P, F, P, I, P, I, I, P],
         "llmx_moe_combine": [P, P, P, P, I, I, I, I, P],
         "llmx_fill_i32": [P, I, L, P],
@@ -158,11 +167,143 @@ def take_launches() -> dict:
 
 
 # ---------------------------------------------------------------------------
-def embed_gather(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor) -> None:
+def embed_gather(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor, scale: float = 1.0) -> None:
+    """out[t] = table[ids[t]] * scale, widened to float32."""
     rows, width = out.shape
     _check(lib().llmx_embed_gather(_dev(table, "table", shape=(table.shape[0], width)), _code(table.dtype),
                                    _dev(ids, "ids", torch.int32, (rows,)), _dev(out, "out", torch.float32),
-                                   rows, width, _stream()), "embed_gather")
+                                   rows, width, float(scale), _stream()), "embed_gather")
+
+
+def rmsnorm_pair(x: torch.Tensor, w1: torch.Tensor, w2: Optional[torch.Tensor], eps: float, out1: torch.Tensor,
+                 out2: Optional[torch.Tensor]) -> None:
+    """Two RMS norms of the same float32 rows with one eps and two gains: out1 = x * (r * w1), out2 = x * (r * w2), r formed
+    once; each output has the bits `rmsnorm` gives with its gain."""
+    rows, n = x.shape
+    if (w2 is None) != (out2 is None) or (out2 is not None and out2.dtype != out1.dtype):
+        raise KernelError("rmsnorm_pair: the second gain and the second output come together, in the first output's type")
+    _check(lib().llmx_rmsnorm_pair(_dev(x, "x", torch.float32), _dev(w1, "w1", torch.float32, (n,)), _dev(w2, "w2", torch.float32, (n,)),
+                                   float(eps), _dev(out1, "out1", shape=(rows, n)), _dev(out2, "out2", shape=(rows, n)), _code(out1.dtype),
+                                   rows, n, _stream()), "rmsnorm_pair")
+
+
+def scale_add(x: torch.Tensor, y1: torch.Tensor, s1: Optional[torch.Tensor], y2: Optional[torch.Tensor] = None,
+              s2: Optional[torch.Tensor] = None, copy: Optional[torch.Tensor] = None) -> None:
+    """x += s1 * y1 (+ s2 * y2), float32 rows and per-feature scales (None: 1); `copy` receives the new rows in its type."""
+    rows, n = x.shape
+    _check(lib().llmx_scale_add(_dev(x, "x", torch.float32), _dev(y1, "y1", torch.float32, (rows, n)), _dev(s1, "s1", torch.float32, (n,)),
+                                _dev(y2, "y2", torch.float32, (rows, n)), _dev(s2 if y2 is not None else None, "s2", torch.float32, (n,)),
+                                _dev(copy, "copy", shape=(rows, n)), _code(copy.dtype) if copy is not None else F32, rows, n, _stream()),
+           "scale_add")
+
+
+def rmsnorm_add(x: torch.Tensor, y: torch.Tensor, weight: torch.Tensor, eps: float) -> None:
+    """x += RMSNorm(y) * weight, all float32."""
+    rows, n = x.shape
+    _check(lib().llmx_rmsnorm_add(_dev(x, "x", torch.float32), _dev(y, "y", torch.float32, (rows, n)), _dev(weight, "weight", torch.float32, (n,)),
+                                  float(eps), rows, n, _stream()), "rmsnorm_add")
+
+
+def act_xielu(z: torch.Tensor, pq: torch.Tensor, out: torch.Tensor) -> None:
+    """out = xIELU(z) with the two numbers pq = (p, q) on the device: z > 0: softplus(p) z^2 + z/2; else (1/2 + softplus(q)) (e^z - 1 - z) + z/2."""
+    if out.shape != z.shape:
+        raise KernelError("act_xielu: shapes do not agree")
+    _check(lib().llmx_act_xielu(_dev(z, "z", torch.float32), _dev(pq, "pq", torch.float32, (2,)), _dev(out, "out"), _code(out.dtype),
+                                z.numel(), _stream()), "act_xielu")
+
+
+def act_gelu_gather(z: torch.Tensor, table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor, col0: int) -> None:
+    """out[t, j] = gelu_tanh(z[t, j]) * table[ids[t], col0 + j]."""
+    rows, n = z.shape
+    if col0 < 0 or col0 + n > table.shape[1]:
+        raise KernelError(f"act_gelu_gather: columns {col0}..{col0 + n} outside the table's {table.shape[1]}")
+    _check(lib().llmx_act_gelu_gather(_dev(z, "z", torch.float32), _dev(table, "table"), _code(table.dtype), _dev(ids, "ids", torch.int32, (rows,)),
+                                      _dev(out, "out", shape=(rows, n)), _code(out.dtype), rows, n, int(col0), table.shape[1], _stream()),
+           "act_gelu_gather")
+
+
+def mingru_scan(zxg: torch.Tensor, bz: Optional[torch.Tensor], bx: Optional[torch.Tensor], state: torch.Tensor, slot_read: torch.Tensor,
+                slot_write: torch.Tensor, entry_rows: torch.Tensor, out: torch.Tensor) -> None:
+    """The minGRU recurrence over each entry's rows (see csrc/recurrent.hip): zxg [T, 3W] float32 pre-activations
+    (gate | candidate | output gate), state [slots, W] float32 read at slot_read[e] and written at slot_write[e],
+    entry_rows [n_entries, 2] (first row, rows); out [T, W] = S_t * silu(g_t)."""
+    T, W3 = zxg.shape
+    W = W3 // 3
+    n_e = entry_rows.shape[0]
+    if W3 != 3 * W or state.shape[1] != W or tuple(out.shape) != (T, W):
+        raise KernelError("mingru_scan: shapes do not agree")
+    _check(lib().llmx_mingru_scan(_dev(zxg, "zxg", torch.float32), _dev(bz, "bz", torch.float32, (W,)), _dev(bx, "bx", torch.float32, (W,)),
+                                  _dev(state, "state", torch.float32), _dev(slot_read, "slot_read", torch.int32, (n_e,)),
+                                  _dev(slot_write, "slot_write", torch.int32, (n_e,)), _dev(entry_rows, "entry_rows", torch.int32, (n_e, 2)),
+                                  _dev(out, "out"), _code(out.dtype), n_e, W, _stream()), "mingru_scan")
+
+
+def latent_prep(proj: torch.Tensor, norm_w: torch.Tensor, cos_sin: torch.Tensor, pos: torch.Tensor, row_entry: torch.Tensor,
+                tables: torch.Tensor, q_plain: torch.Tensor, q_rot: torch.Tensor, cache: torch.Tensor, eps: float, heads: int, dim: int,
+                rot_dim: int, rank: int, write_cache: bool = True) -> None:
+    """From the float32 rows proj = [q of `heads` x (dim | rot_dim) | latent of `rank` | key part of rot_dim | ...]: the
+    queries head by head (q_plain [H, T, dim], q_rot [H, T, rot_dim] rotated), and into the row's cache place the
+    RMS-normed latent and the rotated key part.  cos_sin [positions, dims]: the first `dims` of a rotated part turn as
+    interleaved pairs."""
+    T, ldp = proj.shape
+    n_pages, page_tokens, width = cache.shape
+    dims = cos_sin.shape[1]
+    if width != rank + rot_dim or q_plain.dtype != cache.dtype or q_rot.dtype != cache.dtype:
+        raise KernelError("latent_prep: the cache does not fit the latent and the key part")
+    _check(lib().llmx_latent_prep(_dev(proj, "proj", torch.float32), _dev(norm_w, "norm_w", torch.float32, (rank,)),
+                                  _dev(cos_sin, "cos_sin", torch.float32), _dev(pos, "pos", torch.int32, (T,)),
+                                  _dev(row_entry, "row_entry", torch.int32, (T,)), _dev(tables, "tables", torch.int32),
+                                  _dev(q_plain, "q_plain", shape=(heads, T, dim)), _dev(q_rot, "q_rot", shape=(heads, T, rot_dim)),
+                                  _dev(cache, "cache"), _code(cache.dtype), float(eps), T, ldp, heads, dim, rot_dim, rank, dims, page_tokens,
+                                  tables.shape[1], 1 if write_cache else 0, _stream()), "latent_prep")
+
+
+def latent_attention(q_lat: torch.Tensor, q_rot: torch.Tensor, cache: torch.Tensor, pos: torch.Tensor, row_entry: torch.Tensor,
+                     tables: torch.Tensor, out: torch.Tensor, scale: float, window: int = 0, scratch=None) -> None:
+    """Causal softmax attention of every (head, row) over its request's paged latents: score = (q_lat . c + q_rot . k_rot)
+    * scale, result = sum of weights * c.  q_lat and out [H, T, C], q_rot [H, T, R], cache [pages, page_tokens, C + R].
+    `scratch(name, shape, dtype)`: storage that lives as long as the caller's step."""
+    H, T, C = q_lat.shape
+    R = q_rot.shape[2]
+    n_pages, page_tokens, width = cache.shape
+    if width != C + R or tuple(q_rot.shape[:2]) != (H, T) or out.shape != q_lat.shape or len({q_lat.dtype, q_rot.dtype, cache.dtype, out.dtype}) != 1:
+        raise KernelError("latent_attention: shapes or dtypes do not agree")
+    _check(lib().llmx_latent_attention_generic(_dev(q_lat, "q_lat"), _dev(q_rot, "q_rot"), _dev(cache, "cache"), _dev(pos, "pos", torch.int32, (T,)),
+                                               _dev(row_entry, "row_entry", torch.int32, (T,)), _dev(tables, "tables", torch.int32),
+                                               _dev(out, "out"), _code(q_lat.dtype), float(scale), T, H, C, R, page_tokens, tables.shape[1],
+                                               int(window), _stream()), "latent_attention")
+
+
+def head_gate(values: torch.Tensor, gate: Optional[torch.Tensor], out: torch.Tensor) -> None:
+    """out[t, h*V + d] = sigmoid(gate[t, h]) * values[h, t, d]; gate a float32 view [T, H] whose rows may be strided
+    (columns of a wider projection), or None for no gate."""
+    H, T, V = values.shape
+    ldg = 0
+    addr = 0
+    if gate is not None:
+        if not gate.is_cuda or gate.dtype != torch.float32 or tuple(gate.shape) != (T, H) or gate.stride(1) != 1:
+            raise KernelError("head_gate: the gate is float32 [T, H] on the GPU with unit stride along the heads")
+        ldg, addr = gate.stride(0), gate.data_ptr()
+    _check(lib().llmx_head_gate(_dev(values, "values", torch.float32), addr, ldg, _dev(out, "out", shape=(T, H * V)), _code(out.dtype),
+                                T, H, V, _stream()), "head_gate")
+
+
+_HEAD_GROUPS: dict = {}
+
+
+def head_groups(heads: int, rows: int, device):
+    """What grouped_gemm wants for `heads` groups of `rows` rows each, laid out group by group: (offsets, pairs, active,
+    n_active) on the device.  Cached: a step's launches may be recorded into a graph that reads them later."""
+    key = (heads, rows, str(device))
+    got = _HEAD_GROUPS.get(key)
+    if got is None:
+        if len(_HEAD_GROUPS) > 512:
+            _HEAD_GROUPS.clear()
+        got = _HEAD_GROUPS[key] = (torch.arange(0, (heads + 1) * rows, rows, dtype=torch.int32, device=device),
+                                   torch.arange(heads * rows, dtype=torch.int32, device=device),
+                                   torch.arange(heads, dtype=torch.int32, device=device),
+                                   torch.full((1,), heads, dtype=torch.int32, device=device))
+    return got
 
 
 def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: Optional[torch.Tensor], out32: Optional[torch.Tensor] = None,

@@ -3,7 +3,7 @@
 from .base import (BuildContext, Embedding, FeedForward, Head, LayerCache, Mixer, Norm, Part, PositionEncoding, build_part,
                    register, unregister)
 from .spec import BlockSpec, CacheTensor, KVNeed, ModelSpec, PagedNeed, PartSpec, RunEntry, StateNeed, TensorSpec
-from . import norm, position, attention, moe, embedding, block  # noqa: F401  (registers the built-in parts)
+from . import norm, position, attention, latent_attention, recurrent, moe, embedding, token_input, block  # noqa: F401  (registers the built-in parts)
 
 __all__ = ["BuildContext", "Embedding", "FeedForward", "Head", "LayerCache", "Mixer", "Norm", "Part", "PositionEncoding",
            "build_part", "register", "unregister", "BlockSpec", "CacheTensor", "KVNeed", "PagedNeed", "ModelSpec", "PartSpec", "RunEntry", "StateNeed",

@@ -10,7 +10,10 @@ What a part sees of a step (the `step` argument, an `engine.batch.StepState`):
   step.row_entry                  int32 [T]: index of each row's request among the step's entries
   step.entries                    host list of EntryView(slot, row0, n, past): a request's state slot, its first row,
                                   its number of rows and the tokens it held before the step
-  step.entry_slots                int32 [n_entries] on the device: each entry's state slot
+  step.entry_slots                int32 [n_entries] on the device: each entry's state slot (the one this step writes)
+  step.entry_held_slots           int32 [n_entries] on the device: the slot that holds each entry's state as the step found it
+                                  (another than entry_slots when steps compute into a second slot)
+  step.entry_rows                 int32 [n_entries, 2] on the device: each entry's first row and number of rows
   step.tables(group)              int32 [n_entries, max_blocks]: page ids of each entry in cache group `group`
   step.buf(name, shape, dtype)    a scratch tensor that lives until the step ends (same name, same storage)
   step.shared(key, make)          something a part wants once a step (a kernel's work plan, a second position stream):
@@ -121,6 +124,9 @@ class LayerCache:
 class Mixer(Part):
     #: True when forward wants the normed rows also as float32 (`h32`)
     wants_f32_input = False
+    #: a mixer with state: True when forward reads a request's state at step.entry_held_slots and writes it at
+    #: step.entry_slots, so that the engine need not copy the state into the step's slot before the step
+    steps_between_slots = False
 
     def takes_deferred_norm(self, step) -> bool:
         """Whether, for this step, forward accepts a Norm.deferred() description as h and h32 in place of tensors."""
@@ -163,7 +169,8 @@ class Head(Part):
 
 # ---------------------------------------------------------------------------
 # registries: part name -> class
-_REGISTRIES: Dict[str, Dict[str, Callable]] = {k: {} for k in ("norm", "position", "mixer", "feed_forward", "embedding", "head", "block")}
+_REGISTRIES: Dict[str, Dict[str, Callable]] = {k: {} for k in ("norm", "position", "mixer", "feed_forward", "embedding", "head", "block",
+                                                                 "scale", "token_input")}
 
 
 def register(family: str, kind: str, cls: Callable, replace: bool = False) -> None:

@@ -1,15 +1,19 @@
-"""The arrangement of a layer's parts.
+"""The arrangements of a layer's parts.
 
 "prenorm": x += mixer(norm(x)); x += ffn(norm(x)) with the residual x in float32: the arrangement of
 /root/reference/src/model/arch/minimax_m3.hpp:247-287 (norm, mixer joined into the residual, norm, feed-forward joined).
+"parallel": x += s1 * mixer(norm1(x)) + s2 * ffn(norm2(x)) with both norms of the same x, learned factors s1, s2 a
+coordinate, and an optional per-layer token input after the sum.
 """
 
 from __future__ import annotations
 
 import torch
 
-from .base import BuildContext, LayerCache, build_part, register
-from .spec import BlockSpec
+from .. import ops
+from .base import BuildContext, LayerCache, Mixer, Part, build_part, register
+from .norm import RMSNorm
+from .spec import BlockSpec, TensorSpec
 
 
 class PreNormBlock:
@@ -45,4 +49,79 @@ class PreNormBlock:
         self.ffn.forward(step, h, x, True, h32)
 
 
+class LayerScale(Part):
+    """One learned factor a coordinate on a part's result.  params: width; tensor: the prefix itself, (width,)."""
+    graph_safe = True
+
+    def __init__(self, params, prefix, ctx):
+        super().__init__(params, prefix, ctx)
+        self.width = int(params["width"])
+        self.weight = None
+
+    def tensor_specs(self, available):
+        return [TensorSpec(self.prefix, (self.width,), "norm")]
+
+    def load(self, tensors):
+        self.weight = tensors[self.prefix]
+
+
+class ParallelBlock:
+    """x += s1 * mixer(norm1(x)) + s2 * ffn(norm2(x)), both of the same x, then an optional token input that reads the
+    new x.  The slots: mixer_norm, mixer, and (both or neither) ffn_norm, ffn; in `extra`: "mixer_scale" and "ffn_scale"
+    (family "scale": a factor a coordinate on each result before the sum, optional) and "token_input" (family
+    "token_input", optional).  Two RMS norms with one eps are one pass over x with two gains."""
+    graph_safe = True
+
+    def __init__(self, spec: BlockSpec, ctx: BuildContext):
+        if (spec.ffn is None) != (spec.ffn_norm is None):
+            raise ValueError("parallel block: a feed-forward and its norm come together")
+        self.mixer_norm = build_part("norm", spec.mixer_norm, ctx)
+        self.mixer = build_part("mixer", spec.mixer, ctx)
+        self.ffn_norm = build_part("norm", spec.ffn_norm, ctx) if spec.ffn_norm is not None else None
+        self.ffn = build_part("feed_forward", spec.ffn, ctx) if spec.ffn is not None else None
+        built = {}
+        for slot, family in (("mixer_scale", "scale"), ("ffn_scale", "scale"), ("token_input", "token_input")):
+            if slot in spec.extra:
+                got_family, part = spec.extra[slot]
+                if got_family != family:
+                    raise ValueError(f"parallel block: {slot} is a part of family {family!r}, not {got_family!r}")
+                built[slot] = build_part(family, part, ctx)
+        unknown = set(spec.extra) - {"mixer_scale", "ffn_scale", "token_input"}
+        if unknown:
+            raise ValueError(f"parallel block: no slot named {sorted(unknown)}")
+        self.mixer_scale = built.get("mixer_scale")
+        self.ffn_scale = built.get("ffn_scale") if self.ffn is not None else None
+        self.token_input = built.get("token_input")
+        a, b = self.mixer_norm, self.ffn_norm
+        self._one_pass = isinstance(a, RMSNorm) and (b is None or (isinstance(b, RMSNorm) and b.eps == a.eps and b.width == a.width))
+
+    def parts(self):
+        return [p for p in (self.mixer_norm, self.mixer, self.ffn_norm, self.ffn, self.mixer_scale, self.ffn_scale, self.token_input)
+                if p is not None]
+
+    def forward(self, step, x: torch.Tensor, cache: LayerCache) -> None:
+        T, E = x.shape
+        act = step.act_dtype
+        h1 = step.buf("block.h", (T, E), act)
+        h2 = step.buf("block.h2", (T, E), act) if self.ffn is not None else None
+        if self._one_pass:
+            ops.rmsnorm_pair(x, self.mixer_norm.weight, self.ffn_norm.weight if h2 is not None else None, self.mixer_norm.eps, h1, h2)
+        else:
+            self.mixer_norm.forward(step, x, h1)
+            if h2 is not None:
+                self.ffn_norm.forward(step, x, h2)
+        y1 = step.buf("block.y1", (T, E), torch.float32)
+        self.mixer.forward(step, h1, y1, False, cache)
+        y2 = None
+        if self.ffn is not None:
+            y2 = step.buf("block.y2", (T, E), torch.float32)
+            self.ffn.forward(step, h2, y2, False)
+        copy = step.buf("block.x_act", (T, E), act) if self.token_input is not None else None
+        ops.scale_add(x, y1, self.mixer_scale.weight if self.mixer_scale else None, y2, self.ffn_scale.weight if self.ffn_scale else None, copy)
+        if self.token_input is not None:
+            self.token_input.forward(step, x, copy)
+
+
 register("block", "prenorm", PreNormBlock)
+register("block", "parallel", ParallelBlock)
+register("scale", "layer_scale", LayerScale)

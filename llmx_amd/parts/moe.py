@@ -1,4 +1,5 @@
-"""Feed-forward parts: routed SwiGLU experts behind a scored top-k router, and a dense SwiGLU.
+"""Feed-forward parts: routed SwiGLU experts behind a scored top-k router, a dense SwiGLU, and a dense layer with one
+activation between its two products.
 
 Router: z = h.Wr^T in float32 on unrounded rows (/root/reference/src/backends/backend.hpp:944-947); score sigmoid(z);
 the pick key is score + correction bias, k picks, the lowest id on ties; weight = the unbiased score, divided by the
@@ -139,5 +140,38 @@ class DenseGLU(FeedForward):
         ops.gemm(act, self.w_down, out, ops.EPI_ADD if accumulate else ops.EPI_STORE, scratch=step.buf)
 
 
+class DenseAct(FeedForward):
+    """params: hidden, intermediate, activation ("xielu").  y = W_down act(W_up h); tensors <prefix>up, down, and for xIELU
+    <prefix>act = (p, q): act(z) = softplus(p) z^2 + z/2 for z > 0, (1/2 + softplus(q)) (e^z - 1 - z) + z/2 otherwise."""
+    graph_safe = True
+
+    def __init__(self, params, prefix, ctx):
+        super().__init__(params, prefix, ctx)
+        self.hidden = int(params["hidden"])
+        self.intermediate = int(params["intermediate"])
+        self.activation = str(params.get("activation", "xielu"))
+        if self.activation != "xielu":
+            raise ValueError(f"dense feed-forward: activation {self.activation!r} is not one of ['xielu']")
+        self.w_up = self.w_down = self.act = None
+
+    def tensor_specs(self, available):
+        F, E = self.intermediate, self.hidden
+        return [TensorSpec(self.name("up"), (F, E)), TensorSpec(self.name("down"), (E, F)),
+                TensorSpec(self.name("act"), (2,), "bias", dtype="float32", init=("uniform", -1.0, 1.0))]
+
+    def load(self, tensors):
+        self.w_up = tensors[self.name("up")]
+        self.w_down = tensors[self.name("down")]
+        self.act = tensors[self.name("act")]
+
+    def forward(self, step, h, out, accumulate, h32=None):
+        z = step.buf("dense.pre", (step.rows, self.intermediate), torch.float32)
+        ops.gemm(h, self.w_up, z, scratch=step.buf)
+        a = step.buf("dense.act", (step.rows, self.intermediate), step.act_dtype)
+        ops.act_xielu(z, self.act, a)
+        ops.gemm(a, self.w_down, out, ops.EPI_ADD if accumulate else ops.EPI_STORE, scratch=step.buf)
+
+
 register("feed_forward", "routed_experts", RoutedExperts)
+register("feed_forward", "dense_act", DenseAct)
 register("feed_forward", "dense_glu", DenseGLU)

@@ -16,20 +16,28 @@ from .spec import TensorSpec
 
 
 class RMSNorm(Norm):
-    """params: width, eps; tensor: <prefix>weight (width,)."""
+    """params: width, eps; gain ("vector", the default: one weight a coordinate; "scalar": the file holds one number for
+    all coordinates); tensor (the name's last part, "weight" by default; "" when the prefix is the whole name).
+    Tensor: <prefix><tensor>, (width,) or ()."""
     graph_safe = True
 
     def __init__(self, params, prefix, ctx):
         super().__init__(params, prefix, ctx)
         self.width = int(params["width"])
         self.eps = float(params["eps"])
+        self.gain = str(params.get("gain", "vector"))
+        if self.gain not in ("vector", "scalar"):
+            raise ValueError(f"norm gain {self.gain!r} is not one of ['scalar', 'vector']")
+        self.tensor = str(params.get("tensor", "weight"))
         self.weight: Optional[torch.Tensor] = None
 
     def tensor_specs(self, available):
-        return [TensorSpec(self.name("weight"), (self.width,), "norm")]
+        return [TensorSpec(self.name(self.tensor), (self.width,) if self.gain == "vector" else (), "norm")]
 
     def load(self, tensors):
-        self.weight = tensors[self.name("weight")]
+        w = tensors[self.name(self.tensor)]
+        # one number for all coordinates is kept as a row of that number, which every norm kernel takes as it is
+        self.weight = w if self.gain == "vector" else w.reshape(1).expand(self.width).contiguous()
 
     def forward(self, step, x, out, out32=None, pick=None):
         ops.rmsnorm(x, self.weight, self.eps, out, out32, pick)

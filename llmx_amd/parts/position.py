@@ -56,6 +56,64 @@ class PartialRotary(PositionEncoding):
         return self.cos_sin, self.rotary_dim
 
 
+def blended_frequencies(dims: int, base: float, scaling) -> tuple:
+    """(frequencies [dims/2] float64, magnitude): f_i = base^(-2i/dims); with `scaling` = {factor, original, fast, slow}
+    the YaRN blend: pairs that turn more than `fast` times over `original` positions keep f_i, pairs that turn fewer
+    than `slow` times get f_i / factor, and between them a linear ramp over the pair index decides:
+    pair(t) = dims ln(original / (2 pi t)) / (2 ln base), lo = max(floor(pair(fast)), 0), hi = min(ceil(pair(slow)),
+    dims - 1), ramp_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1), f = f_i / factor * ramp_i + f_i (1 - ramp_i);
+    cos and sin are then multiplied by magnitude = 0.1 ln(factor) + 1."""
+    i = np.arange(dims // 2, dtype=np.float64)
+    f = np.power(float(base), -2.0 * i / float(dims)) if dims else i
+    if not scaling:
+        return f, 1.0
+    factor, original = float(scaling["factor"]), float(scaling["original"])
+    fast, slow = float(scaling["fast"]), float(scaling["slow"])
+    if not (factor > 0.0 and original > 0.0 and fast > 0.0 and slow > 0.0 and base > 1.0):
+        raise ValueError("rotary scaling: factor, original, fast and slow must be positive and the base above 1")
+
+    def pair_of(turns: float) -> float:
+        return dims * np.log(original / (2.0 * np.pi * turns)) / (2.0 * np.log(float(base)))
+
+    lo = max(int(np.floor(pair_of(fast))), 0)
+    hi = min(int(np.ceil(pair_of(slow))), dims - 1)
+    ramp = np.clip((i - lo) / max(hi - lo, 0.001), 0.0, 1.0)
+    return f / factor * ramp + f * (1.0 - ramp), 0.1 * float(np.log(factor)) + 1.0
+
+
+def scaled_table(positions: int, dims: int, base: float, scaling) -> np.ndarray:
+    """[positions, dims] float32: magnitude * cos of the dims/2 pairs' angles, then magnitude * sin.  The angle is the
+    float32 product of the position and the float32 frequency; cos and sin are evaluated in float64 on it and rounded
+    once, as `neox_table` does."""
+    if dims == 0:
+        return np.zeros((positions, 0), dtype=np.float32)
+    f, magnitude = blended_frequencies(dims, base, scaling)
+    pos = np.arange(positions, dtype=np.float32)[:, None]
+    angle = (pos * f.astype(np.float32)[None, :]).astype(np.float32).astype(np.float64)
+    return (np.concatenate([np.cos(angle), np.sin(angle)], axis=1) * magnitude).astype(np.float32)
+
+
+class ScaledRotary(PositionEncoding):
+    """Rotary pairs with an optional YaRN blend of the frequencies.  params: dims (even; the rotated dims), base, scaling
+    (None, or {factor, original, fast, slow}), pairing ("interleaved", the default here: dims 2i and 2i + 1; "halves")."""
+    graph_safe = True
+
+    def __init__(self, params, prefix, ctx):
+        super().__init__(params, prefix, ctx)
+        self.pairing = str(params.get("pairing", "interleaved"))
+        if self.pairing not in PAIRINGS:
+            raise ValueError(f"rotary pairing {self.pairing!r} is not one of {sorted(PAIRINGS)}")
+        self.rotary_dim = int(params["dims"])
+        if self.rotary_dim % 2 or self.rotary_dim < 0:
+            raise ValueError(f"rotary width {self.rotary_dim} must be even")
+        self.base = float(params["base"])
+        self.scaling = dict(params["scaling"]) if params.get("scaling") else None
+        self.cos_sin = torch.from_numpy(scaled_table(ctx.max_positions, self.rotary_dim, self.base, self.scaling)).to(ctx.device)
+
+    def rotation(self):
+        return self.cos_sin, self.rotary_dim
+
+
 class NoPosition(PositionEncoding):
     """Leaves rows as they are."""
     graph_safe = True
@@ -69,4 +127,5 @@ class NoPosition(PositionEncoding):
 
 
 register("position", "rotary_neox_partial", PartialRotary)
+register("position", "rotary_scaled", ScaledRotary)
 register("position", "none", NoPosition)

@@ -68,8 +68,8 @@ class BlockSpec:
     """
     mixer_norm: PartSpec
     mixer: PartSpec
-    ffn_norm: PartSpec
-    ffn: PartSpec
+    ffn_norm: Optional[PartSpec] = None     # None (with ffn None): a layer without a feed-forward, where the arrangement has such
+    ffn: Optional[PartSpec] = None
     arrangement: str = "prenorm"
     extra: Dict[str, Tuple[str, PartSpec]] = field(default_factory=dict)   # name -> (family, part)
 

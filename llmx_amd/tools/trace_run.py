@@ -33,7 +33,7 @@ def main(argv=None) -> int:
     ap.add_argument("--max-tokens", type=int, required=True,
                     help="most tokens live requests hold at any time, each request's count rounded up to a multiple of 64")
     ap.add_argument("--page-tokens", type=int, default=16, help="tokens a cache page holds")
-    ap.add_argument("--max-requests", type=int, default=8, help="most requests live at a time")
+    ap.add_argument("--max-requests", type=int, default=4, help="most requests live at a time (the state slots the engine makes)")
     ap.add_argument("--routing", action="store_true", help="also write every step's expert picks and router logits")
     args = ap.parse_args(argv)
     if args.max_tokens <= 0:
