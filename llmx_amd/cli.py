@@ -371,7 +371,7 @@ def cmd_random(a) -> int:
 
 
 def build_parser():
-    ap = argparse.ArgumentParser(prog="llmx", description="MiniMax-M3 on one MI355X: generate, logits, perplexity, replay, random, bench")
+    ap = argparse.ArgumentParser(prog="llmx", description="llmx_amd on one MI355X (MiniMax-M3, Nenotar): generate, logits, perplexity, replay, random, bench")
     sub = ap.add_subparsers(dest="command", required=True)
     g = sub.add_parser("generate", help="generate tokens after a prompt of token ids")
     g.add_argument("words", nargs="*", metavar="MODEL [PROMPT]",

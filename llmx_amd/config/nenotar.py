@@ -96,6 +96,11 @@ class NenotarConfig:
         r.finish((), ARCHITECTURE)
         return cfg
 
+    @property
+    def vocab_size(self) -> int:
+        """The vocabulary under the name the command line asks every configuration for."""
+        return self.vocab
+
     def to_json(self) -> dict:
         layers = []
         for layer in self.layers:
