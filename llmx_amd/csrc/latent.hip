@@ -21,6 +21,7 @@ struct LatentPrepArgs {
     void* q_plain;
     void* q_rot;
     void* cache;
+    void* cache_t;          // null, or a second copy of the latents [pages, C, page_tokens] (transposed within the page)
     float eps;
     int T, ldp, H, D, R, C, dims, page_tokens, max_blocks, write_cache;
 };
@@ -67,17 +68,22 @@ __global__ void __launch_bounds__(256) latent_prep_kernel(LatentPrepArgs a) {
     const float r = 1.0f / sqrtf(s / (float)a.C + a.eps);
     const int page = a.tables[(size_t)a.row_entry[t] * a.max_blocks + p / a.page_tokens];
     TC* out = (TC*)a.cache + ((size_t)page * a.page_tokens + p % a.page_tokens) * (a.C + a.R);
-    for (int i = threadIdx.x; i < a.C; i += 256) st(out + i, lat[i] * (r * a.norm_w[i]));
+    TC* out_t = a.cache_t ? (TC*)a.cache_t + (size_t)page * a.C * a.page_tokens + p % a.page_tokens : nullptr;
+    for (int i = threadIdx.x; i < a.C; i += 256) {
+        const float c = lat[i] * (r * a.norm_w[i]);
+        st(out + i, c);
+        if (out_t) st(out_t + (size_t)i * a.page_tokens, c);
+    }
     for (int i = threadIdx.x; i < a.R; i += 256) st(out + a.C + i, rotated_interleaved(lat + a.C, cs, i, a.dims));
 }
 
 extern "C" int llmx_latent_prep(const float* proj, const float* norm_w, const float* cos_sin, const int* pos, const int* row_entry,
-                                const int* tables, void* q_plain, void* q_rot, void* cache, int dtype, float eps, int T, int ldp, int H, int D,
+                                const int* tables, void* q_plain, void* q_rot, void* cache, void* cache_t, int dtype, float eps, int T, int ldp, int H, int D,
                                 int R, int C, int dims, int page_tokens, int max_blocks, int write_cache, hipStream_t stream) {
     if (T <= 0) return 0;
     if (dims % 2 || dims > R || D + R <= 0 || C <= 0 || H * (D + R) + C + R > ldp) return -2;
     llmx_note_launch(LK_LATENT_PREP);
-    LatentPrepArgs a{proj, norm_w, cos_sin, pos, row_entry, tables, q_plain, q_rot, cache, eps, T, ldp, H, D, R, C, dims, page_tokens, max_blocks, write_cache};
+    LatentPrepArgs a{proj, norm_w, cos_sin, pos, row_entry, tables, q_plain, q_rot, cache, cache_t, eps, T, ldp, H, D, R, C, dims, page_tokens, max_blocks, write_cache};
     if (dtype == LLMX_F32) hipLaunchKernelGGL((latent_prep_kernel<float, float>), dim3(T, 2), dim3(256), 0, stream, a);
     else hipLaunchKernelGGL((latent_prep_kernel<bf16_t, bf16_t>), dim3(T, 2), dim3(256), 0, stream, a);
     return LLMX_CHECK_LAUNCH();

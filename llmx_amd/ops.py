@@ -60,7 +60,9 @@ def _declare(h) -> None:
         "llmx_act_xielu": [P, P, P, I, L, P],
         "llmx_act_gelu_gather": [P, P, I, P, P, I, I, I, I, I, P],
         "llmx_mingru_scan": [P, P, P, P, P, P, P, P, I, I, I, P],
-        "llmx_latent_prep": [P, P, P, P, P, P, P, P, P, I, F, I, I, I, I, I, I, I, I, I, I, P],
+        "llmx_latent_prep": [P, P, P, P, P, P, P, P, P, P, I, F, I, I, I, I, I, I, I, I, I, I, P],
+        "llmx_latent_attention_mfma": [P, P, P, P, P, P, P, P, I, P, F, I, I, I, I, I, I, P],
+        "llmx_latent_attention_mfma_ok": [I, I, I],
         "llmx_latent_attention_generic": [P, P, P, P, P, P, P, I, F, I, I, I, I, I, I, I, P],
         "llmx_head_gate": [P, P, I, P, I, I, I, I, P],
         "llmx_rmsnorm": [P, P, P, F, P, I, P, I, I, P],
@@ -240,38 +242,89 @@ def mingru_scan(zxg: torch.Tensor, bz: Optional[torch.Tensor], bx: Optional[torc
 
 def latent_prep(proj: torch.Tensor, norm_w: torch.Tensor, cos_sin: torch.Tensor, pos: torch.Tensor, row_entry: torch.Tensor,
                 tables: torch.Tensor, q_plain: torch.Tensor, q_rot: torch.Tensor, cache: torch.Tensor, eps: float, heads: int, dim: int,
-                rot_dim: int, rank: int, write_cache: bool = True) -> None:
+                rot_dim: int, rank: int, write_cache: bool = True, cache_t: Optional[torch.Tensor] = None) -> None:
     """From the float32 rows proj = [q of `heads` x (dim | rot_dim) | latent of `rank` | key part of rot_dim | ...]: the
     queries head by head (q_plain [H, T, dim], q_rot [H, T, rot_dim] rotated), and into the row's cache place the
     RMS-normed latent and the rotated key part.  cos_sin [positions, dims]: the first `dims` of a rotated part turn as
-    interleaved pairs."""
+    interleaved pairs.  `cache_t` [pages, rank, page_tokens]: a second copy of the latent, transposed within the page."""
     T, ldp = proj.shape
     n_pages, page_tokens, width = cache.shape
     dims = cos_sin.shape[1]
+    if cache_t is not None and (tuple(cache_t.shape) != (n_pages, rank, page_tokens) or cache_t.dtype != cache.dtype):
+        raise KernelError("latent_prep: the transposed copy does not fit the cache")
     if width != rank + rot_dim or q_plain.dtype != cache.dtype or q_rot.dtype != cache.dtype:
         raise KernelError("latent_prep: the cache does not fit the latent and the key part")
     _check(lib().llmx_latent_prep(_dev(proj, "proj", torch.float32), _dev(norm_w, "norm_w", torch.float32, (rank,)),
                                   _dev(cos_sin, "cos_sin", torch.float32), _dev(pos, "pos", torch.int32, (T,)),
                                   _dev(row_entry, "row_entry", torch.int32, (T,)), _dev(tables, "tables", torch.int32),
                                   _dev(q_plain, "q_plain", shape=(heads, T, dim)), _dev(q_rot, "q_rot", shape=(heads, T, rot_dim)),
-                                  _dev(cache, "cache"), _code(cache.dtype), float(eps), T, ldp, heads, dim, rot_dim, rank, dims, page_tokens,
+                                  _dev(cache, "cache"), _dev(cache_t, "cache_t"), _code(cache.dtype), float(eps), T, ldp, heads, dim, rot_dim, rank, dims, page_tokens,
                                   tables.shape[1], 1 if write_cache else 0, _stream()), "latent_prep")
 
 
 def latent_attention(q_lat: torch.Tensor, q_rot: torch.Tensor, cache: torch.Tensor, pos: torch.Tensor, row_entry: torch.Tensor,
-                     tables: torch.Tensor, out: torch.Tensor, scale: float, window: int = 0, scratch=None) -> None:
+                     tables: torch.Tensor, out: torch.Tensor, scale: float, window: int = 0, scratch=None,
+                     cache_t: Optional[torch.Tensor] = None, plan: Optional["LatentPlan"] = None) -> None:
     """Causal softmax attention of every (head, row) over its request's paged latents: score = (q_lat . c + q_rot . k_rot)
     * scale, result = sum of weights * c.  q_lat and out [H, T, C], q_rot [H, T, R], cache [pages, page_tokens, C + R].
-    `scratch(name, shape, dtype)`: storage that lives as long as the caller's step."""
+    `scratch(name, shape, dtype)`: storage that lives as long as the caller's step.  With `cache_t` (the latents once
+    more, [pages, C, page_tokens]) and a `plan` (latent_plan) the matrix-core kernel runs, where latent_attention_mfma_ok
+    says it can; otherwise the universal kernel."""
     H, T, C = q_lat.shape
     R = q_rot.shape[2]
     n_pages, page_tokens, width = cache.shape
     if width != C + R or tuple(q_rot.shape[:2]) != (H, T) or out.shape != q_lat.shape or len({q_lat.dtype, q_rot.dtype, cache.dtype, out.dtype}) != 1:
         raise KernelError("latent_attention: shapes or dtypes do not agree")
+    if cache_t is not None and plan is not None and window == 0 and latent_attention_mfma_ok(q_lat.dtype, C, R, page_tokens):
+        if plan.heads != H or plan.rows != T or tuple(cache_t.shape) != (n_pages, C, page_tokens) or cache_t.dtype != cache.dtype:
+            raise KernelError("latent_attention: the plan or the transposed copy does not fit the step")
+        _check(lib().llmx_latent_attention_mfma(_dev(q_lat, "q_lat"), _dev(q_rot, "q_rot"), _dev(cache, "cache"), _dev(cache_t, "cache_t"),
+                                                _dev(pos, "pos", torch.int32, (T,)), _dev(row_entry, "row_entry", torch.int32, (T,)),
+                                                _dev(tables, "tables", torch.int32), _dev(plan.items, "items", torch.int32), plan.n_items,
+                                                _dev(out, "out"), float(scale), T, H, C, R, page_tokens, tables.shape[1], _stream()),
+               "latent_attention_mfma")
+        return
     _check(lib().llmx_latent_attention_generic(_dev(q_lat, "q_lat"), _dev(q_rot, "q_rot"), _dev(cache, "cache"), _dev(pos, "pos", torch.int32, (T,)),
                                                _dev(row_entry, "row_entry", torch.int32, (T,)), _dev(tables, "tables", torch.int32),
                                                _dev(out, "out"), _code(q_lat.dtype), float(scale), T, H, C, R, page_tokens, tables.shape[1],
                                                int(window), _stream()), "latent_attention")
+
+
+def latent_attention_mfma_ok(dtype: torch.dtype, rank: int, rot_dim: int, page_tokens: int) -> bool:
+    return dtype == torch.bfloat16 and bool(lib().llmx_latent_attention_mfma_ok(int(rank), int(rot_dim), int(page_tokens)))
+
+
+class LatentPlan:
+    """Work items of the matrix-core latent attention for one step's rows: each up to 16 (row, head) columns of one request.
+    It holds no positions, so one plan serves every step with the same rows a request."""
+
+    def __init__(self, items, heads, rows, device):
+        import numpy as np
+        self.heads, self.rows, self.n_items = heads, rows, len(items)
+        self.items = torch.tensor(np.asarray(items, dtype=np.int32).reshape(-1, 4), device=device)
+
+
+_LATENT_PLANS: dict = {}
+
+
+def latent_plan(row_counts, heads: int, device) -> LatentPlan:
+    """row_counts[i]: rows of entry i (entries' rows are consecutive, in order).  With 16 heads or more an item is one row and
+    up to 16 of its heads; with fewer, 16 // heads consecutive rows of one entry with all their heads.  Later rows (longer
+    key ranges) come first."""
+    key = (tuple(row_counts), heads, str(device))
+    plan = _LATENT_PLANS.get(key)
+    if plan is None:
+        items, row0 = [], 0
+        per = max(1, 16 // heads)
+        for n in row_counts:
+            for r in range(((n - 1) // per) * per, -1, -per):
+                for h0 in range(0, heads, 16):
+                    items.append([row0 + r, min(per, n - r), h0, min(16, heads - h0)])
+            row0 += n
+        if len(_LATENT_PLANS) > 256:
+            _LATENT_PLANS.clear()
+        plan = _LATENT_PLANS[key] = LatentPlan(items, heads, row0, device)
+    return plan
 
 
 def head_gate(values: torch.Tensor, gate: Optional[torch.Tensor], out: torch.Tensor) -> None:

@@ -61,8 +61,17 @@ class LatentAttention(Mixer):
         self.gate_width = self.heads if self.gate else 0
         self.w_in = self.w_o = self.latent_norm = self.w_uk_t = self.w_uv = None
 
+    def _matrix_cores(self) -> bool:
+        """Whether this engine's steps run the attention on the matrix cores, which read the latents once more, transposed."""
+        page = self.ctx.page_tokens
+        return bool(page) and self.window is None and self.ctx.device.type == "cuda" \
+            and ops.latent_attention_mfma_ok(self.ctx.act_dtype, self.rank, self.rot_dim, page)
+
     def cache_need(self):
-        return PagedNeed((CacheTensor("latent", (self.down_width,), None, 0),), self.window)
+        tensors = [CacheTensor("latent", (self.down_width,), None, 0)]       # a page: [tokens, kv_rank + rot_dim]
+        if self._matrix_cores():
+            tensors.append(CacheTensor("latent_t", (self.rank,), None, 1))     # the latents once more: [kv_rank, tokens]
+        return PagedNeed(tuple(tensors), self.window)
 
     def tensor_specs(self, available):
         E, q, d, g = self.hidden, self.q_width, self.down_width, self.gate_width
@@ -88,8 +97,14 @@ class LatentAttention(Mixer):
     def _groups(self, step):
         return ops.head_groups(self.heads, step.rows, step.device)
 
+    def _plan(self, step):
+        if not self._matrix_cores():
+            return None
+        return step.shared(("latent.plan", self.heads), lambda: ops.latent_plan([e.n for e in step.entries], self.heads, step.device))
+
     def graph_key(self, step):
-        return self._groups(step)      # a recorded step reads the groups' lists; the key keeps them alive
+        # a recorded step reads the groups' lists and the plan's items; the key keeps them alive
+        return self._groups(step), self._plan(step)
 
     def forward(self, step, h, out, accumulate, cache: LayerCache, h32=None):
         T, H, act = step.rows, self.heads, step.act_dtype
@@ -100,14 +115,14 @@ class LatentAttention(Mixer):
         latents = cache.tensors["latent"]
         tables = step.tables(cache.group)
         ops.latent_prep(proj, self.latent_norm, self.position.rotation()[0], step.positions, step.row_entry, tables, q_plain, q_rot,
-                        latents, self.eps, H, self.dim, self.rot_dim, self.rank, write_cache=cache.writes)
+                        latents, self.eps, H, self.dim, self.rot_dim, self.rank, write_cache=cache.writes, cache_t=cache.tensors.get("latent_t"))
         offsets, pairs, active, n_active = self._groups(step)
         q_lat = step.buf("latent.q_lat", (H, T, self.rank), act)
         ops.grouped_gemm(q_plain.view(H * T, self.dim), self.w_uk_t, q_lat.view(H * T, self.rank), offsets, pairs, 1, ops.EPI_STORE,
                          active, n_active, token_rows=T)
         mixed = step.buf("latent.mixed", (H, T, self.rank), act)
         ops.latent_attention(q_lat, q_rot, latents, step.positions, step.row_entry, tables, mixed, self.scale, window=int(self.window or 0),
-                             scratch=step.buf)
+                             scratch=step.buf, cache_t=cache.tensors.get("latent_t"), plan=self._plan(step))
         values = step.buf("latent.values", (H, T, self.vdim), torch.float32)
         ops.grouped_gemm(mixed.view(H * T, self.rank), self.w_uv, values.view(H * T, self.vdim), offsets, pairs, 1, ops.EPI_STORE,
                          active, n_active, token_rows=T)

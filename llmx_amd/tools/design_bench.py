@@ -1,0 +1,170 @@
+"""Prefill and decode throughput of one design beside the closest other one at equal size, with random weights.
+
+`python bench.py --design nenotar` measures, at sizes that resemble a real model's layers, a Nenotar (latent attention
+and minGRU layers in turn, each with a dense xIELU feed-forward and a per-layer token input) and a MiniMax-M3 of the
+same width, layers, heads and vocabulary whose routed experts hold the same active weights a token: one 2,048-token
+prompt from an empty cache, and decode steps of 1 and 8 requests at a context of 4,096 tokens.  Each record has tok/s,
+ms, the bytes a decode step must read (every weight once and the live cache) with their share of 8 TB/s, and a prompt's
+floating-point work with its share of the bf16 peak.  One JSON line.
+"""
+
+from __future__ import annotations
+
+import json
+import time
+
+HBM_PEAK_GBS = 8000.0
+BF16_PEAK = 2.5e15
+PROMPT = 2048
+CONTEXT = 4096
+
+# name -> (width, layers, heads, ff, recurrent width, token-input dim, vocab); a head is 128 unrotated + 64 rotated dims
+# over a latent of 512, values of 128
+SIZES = {
+    "w2048": (2048, 8, 16, 8192, 3072, 128, 32768),
+    "w4096": (4096, 4, 32, 16384, 6144, 256, 32768),
+}
+
+
+def nenotar_config(width, layers, heads, ff, recurrent, side, vocab):
+    from llmx_amd import NenotarConfig
+    from llmx_amd.config.nenotar import LatentAttentionConfig, LayerConfig, MinGRUConfig, RotaryScaling
+    latent = LatentAttentionConfig(heads=heads, dim=128, rot_dim=64, vdim=128, kv_rank=512, scale=192 ** -0.5, rot_base=10000.0, rot_dims=64,
+                                   rot_scaling=RotaryScaling(40.0, 4096.0, 32.0, 1.0))
+    kinds = [LayerConfig("latent_attention", latent, ff) if i % 2 == 0 else LayerConfig("mingru", MinGRUConfig(recurrent), ff) for i in range(layers)]
+    return NenotarConfig(vocab=vocab, width=width, embedding_scale=1.0, norm_eps=1e-6, layers=tuple(kinds), token_side_dim=side)
+
+
+def closest_config(width, layers, heads, ff, recurrent, side, vocab):
+    """MiniMax-M3 of the same width, layers, heads and vocabulary: 8 experts of which 2 a token, holding together the
+    active weights of the dense feed-forward (2 x width x ff = 2 x 3 x width x intermediate)."""
+    from llmx_amd import MiniMaxM3Config
+    inter = max(64, (ff // 3) // 64 * 64)
+    return MiniMaxM3Config(vocab_size=vocab, hidden_size=width, num_hidden_layers=layers, num_attention_heads=heads, num_key_value_heads=max(1, heads // 4),
+                           head_dim=128, rotary_dim=64, rope_theta=1e6, rms_norm_eps=1e-6, num_local_experts=8, num_experts_per_tok=2,
+                           intermediate_size=inter, routed_scaling_factor=1.0, norm_topk_prob=True, tie_word_embeddings=False,
+                           max_position_embeddings=2 * CONTEXT)
+
+
+def _ids(n, vocab, seed):
+    x, out = (seed * 2654435761 + 1) & 0xFFFFFFFF, []
+    for _ in range(n):
+        x = (x * 1664525 + 1013904223) & 0xFFFFFFFF
+        out.append((x >> 8) % vocab)
+    return out
+
+
+def cache_bytes_a_token(engine) -> int:
+    """Bytes of paged cache one token of one request holds over all layers."""
+    return sum(t.shape[0] * (t.numel() // (t.shape[0] * t.shape[1]) // engine.page_tokens) * t.element_size()
+               for arenas in engine._paged for t in arenas.values())
+
+
+def prompt_flops(engine, T) -> float:
+    """Multiply-adds x 2 of a T-token prompt: every weight matrix once a row (the head for one row), and the attention
+    layers' score and value products over the causal half."""
+    cfg = engine.config
+    weights = sum(v.numel() for p in engine.model.parts() for v in vars(p).values()
+                  if hasattr(v, "numel") and hasattr(v, "dim") and v.dim() >= 2 and v.dtype.is_floating_point)
+    vocab = engine.spec.vocab_size
+    dense = 2.0 * T * (weights - 2 * vocab * engine.spec.hidden_size) + 2.0 * vocab * engine.spec.hidden_size
+    if hasattr(cfg, "num_local_experts"):      # only the picked experts work
+        expert = 3 * cfg.hidden_size * cfg.intermediate_size
+        dense -= 2.0 * T * cfg.num_hidden_layers * (cfg.num_local_experts - cfg.num_experts_per_tok) * expert
+        attn = cfg.num_hidden_layers * 4.0 * cfg.num_attention_heads * cfg.head_dim * T * (T + 1) / 2
+    else:
+        attn = 0.0
+        for layer in cfg.layers:
+            if layer.type == "latent_attention":
+                m = layer.mixer
+                attn += 2.0 * m.heads * (2 * m.kv_rank + m.rot_dim) * T * (T + 1) / 2     # over the latents themselves
+                dense -= 0.0
+        side = getattr(cfg, "token_side_dim", None) or 0
+        dense -= 2.0 * T * vocab * side * len(cfg.layers)                                   # the token table is read, not multiplied
+    return dense + attn
+
+
+def measure(engine, torch, steps, warmup):
+    from llmx_amd import ops
+    from llmx_amd.engine import StepEntry
+    vocab = engine.spec.vocab_size
+    out = torch.empty(8, dtype=torch.int32, device=engine.device)
+    rec = {"weights_gb": round(engine.weight_bytes() / 1e9, 2)}
+    times = []
+    for rep in range(3):
+        rid = f"p{rep}"
+        engine.add_request(rid)
+        ids = _ids(PROMPT, vocab, 500 + rep)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        logits = engine.step([StepEntry(rid, ids, [PROMPT - 1])])
+        ops.argmax_rows(logits, out[:1])
+        out[:1].tolist()
+        torch.cuda.synchronize()
+        times.append(time.perf_counter() - t0)
+        engine.end_request(rid)
+    t = min(times[1:])
+    flops = prompt_flops(engine, PROMPT)
+    rec.update(prefill_tok_s=round(PROMPT / t, 1), prefill_ms=round(t * 1e3, 3), prefill_tflop=round(flops / 1e12, 2),
+               prefill_frac=round(flops / t / BF16_PEAK, 4))
+    for batch in (1, 8):
+        start = CONTEXT - steps - warmup
+        rids = [f"d{batch}_{i}" for i in range(batch)]
+        for i, rid in enumerate(rids):
+            engine.add_request(rid)
+            ids = _ids(start, vocab, 100 + i)
+            for s in range(0, start, PROMPT):
+                engine.step([StepEntry(rid, ids[s:s + PROMPT], [])])
+        last = [_ids(1, vocab, 7 + i)[0] for i in range(batch)]
+
+        def one():
+            nonlocal last
+            logits = engine.step([StepEntry(rid, [t], [0]) for rid, t in zip(rids, last)])
+            ops.argmax_rows(logits, out[:batch])
+            last = out[:batch].tolist()
+
+        for _ in range(warmup):
+            one()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            one()
+        torch.cuda.synchronize()
+        dt = (time.perf_counter() - t0) / steps
+        for rid in rids:
+            engine.end_request(rid)
+        need = engine.weight_bytes() + batch * (CONTEXT - steps / 2) * cache_bytes_a_token(engine)
+        cfg = engine.config
+        if hasattr(cfg, "num_local_experts"):   # of the experts at most batch x picks are read
+            unread = max(0, cfg.num_local_experts - batch * cfg.num_experts_per_tok)
+            need -= cfg.num_hidden_layers * unread * 3 * cfg.hidden_size * cfg.intermediate_size * 2
+        side = getattr(cfg, "token_side_dim", None) or 0
+        need -= 2 * vocab * side * (len(cfg.layers) if side else 0)     # of the token table a step reads its rows only
+        need -= 2 * vocab * engine.spec.hidden_size                     # and of the embedding
+        rec.update({f"decode_b{batch}_tok_s": round(batch / dt, 2), f"decode_b{batch}_ms": round(dt * 1e3, 4),
+                    f"decode_b{batch}_gb": round(need / 1e9, 3), f"decode_b{batch}_frac": round(need / dt / 1e9 / HBM_PEAK_GBS, 4)})
+    return rec
+
+
+def run(design: str, steps: int, warmup: int, sizes=None) -> dict:
+    import torch
+    from llmx_amd import Engine, RandomInit
+    if design != "nenotar":
+        raise SystemExit(f"bench: no design named {design!r} (known: nenotar)")
+    result = {"design": "Nenotar", "closest": "MiniMax-M3 (GQA attention, routed SwiGLU experts)", "dtype": "bf16", "prompt": PROMPT,
+              "context": CONTEXT, "data": "synthetic: LCG token ids, N(0,0.02) weights generated on the device", "sizes": {}}
+    for name in (sizes or SIZES):
+        shape = SIZES[name]
+        per = {}
+        for which, make in (("nenotar", nenotar_config), ("closest", closest_config)):
+            engine = Engine.from_random(make(*shape), RandomInit(seed=0, std=0.02), dtype="bfloat16", kv_tokens=8 * CONTEXT + 4 * PROMPT,
+                                        page_tokens=16, max_requests=8)
+            per[which] = measure(engine, torch, steps, max(2, warmup))
+            del engine
+            torch.cuda.empty_cache()
+        result["sizes"][name] = per
+    return result
+
+
+def main(design: str, steps: int, warmup: int, sizes=None) -> None:
+    print(json.dumps(run(design, steps, warmup, sizes)))

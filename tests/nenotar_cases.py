@@ -53,7 +53,7 @@ CONFIG_Q = {
 CONFIG_R = {
     "architecture": "Nenotar", "vocab": 128, "width": 64, "embedding": {"scale": 3.0}, "norm": {"eps": 1e-6}, "token_side": {"dim": 1},
     "layers": [
-        _layer("latent_attention", _latent(18, 16, 16, 16, 32, 0.18, 10000.0, 16, (4.0, 128, 32.0, 1.0)), 48),
+        _layer("latent_attention", _latent(18, 16, 16, 16, 48, 0.18, 10000.0, 16, (4.0, 128, 32.0, 1.0)), 48),
         _layer("latent_attention", _latent(4, 32, 32, 24, 64, 0.125, 50000.0, 32), 48),
     ],
 }

@@ -167,6 +167,9 @@ def _latent_case(seed, H, D, R, V, C, dims, scaling, positions, page, dtype, sha
     tables[1, :n_pages] = torch.tensor(order, dtype=torch.int32)           # the request is entry 1 of its steps
     tables = dev(tables)
     cache = torch.zeros(n_pages, page, C + R, dtype=dtype, device="cuda")
+    # where the matrix cores take the sizes they run (with the latents' second, transposed copy and a plan of work items)
+    cores = o.latent_attention_mfma_ok(dtype, C, R, page)
+    cache_t = torch.zeros(n_pages, C, page, dtype=dtype, device="cuda") if cores else None
     cos_sin = dev(torch.from_numpy(scaled_table(n_ctx, dims, 300.0, m["rot"].get("scaling"))))
     w_in = torch.cat([w["a.q"], w["a.dkv"], w["a.g"]])
     uk_t = dev(w["a.uk"].view(H, D, C).transpose(1, 2), dtype)
@@ -181,10 +184,13 @@ def _latent_case(seed, H, D, R, V, C, dims, scaling, positions, page, dtype, sha
         pos = dev(torch.tensor(rows, dtype=torch.int32))
         entry = dev(torch.ones(T, dtype=torch.int32))
         q_plain, q_rot = torch.empty(H, T, D, dtype=dtype, device="cuda"), torch.empty(H, T, R, dtype=dtype, device="cuda")
-        o.latent_prep(proj, dev(w["a.dkv.norm"]), cos_sin, pos, entry, tables, q_plain, q_rot, cache, 1e-6, H, D, R, C)
+        o.latent_prep(proj, dev(w["a.dkv.norm"]), cos_sin, pos, entry, tables, q_plain, q_rot, cache, 1e-6, H, D, R, C, cache_t=cache_t)
         q_lat = torch.bmm(q_plain.float(), uk_t.float().transpose(1, 2)).to(dtype).contiguous()
         mixed = torch.empty(H, T, C, dtype=dtype, device="cuda")
-        o.latent_attention(q_lat, q_rot, cache, pos, entry, tables, mixed, 0.3)
+        o.take_launches()
+        o.latent_attention(q_lat, q_rot, cache, pos, entry, tables, mixed, 0.3, cache_t=cache_t,
+                           plan=o.latent_plan([0, T], H, "cuda") if cores else None)
+        assert ("latent_attention.mfma" in o.take_launches()) == cores
         values = torch.bmm(mixed.float(), uv.float().transpose(1, 2)).contiguous()
         joined = torch.empty(T, H * V, dtype=dtype, device="cuda")
         o.head_gate(values, proj[:, H * (D + R) + C + R:], joined)
@@ -195,7 +201,8 @@ def _latent_case(seed, H, D, R, V, C, dims, scaling, positions, page, dtype, sha
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["float32", "bfloat16"])
 @pytest.mark.parametrize("sizes", [(3, 24, 16, 40, 48, 16, (8.0, 64, 16.0, 2.0)), (1, 5, 6, 3, 10, 4, None), (17, 8, 0, 8, 16, 0, None),
-                                   (2, 16, 8, 24, 130, 8, (2.0, 16, 4.0, 1.5))], ids=["even", "ragged", "no_rotation", "wide_latent"])
+                                   (2, 16, 8, 24, 130, 8, (2.0, 16, 4.0, 1.5)), (20, 16, 32, 8, 96, 32, None), (16, 8, 64, 8, 512, 64, None)],
+                         ids=["even", "ragged", "no_rotation", "wide_latent", "twenty_heads", "real_latent"])
 def test_latent_attention_rows_at_page_borders_and_first_tokens(dtype, sizes):
     H, D, R, V, C, dims, scaling = sizes
     positions = [0, 1, 2, 15, 16, 17, 63, 64, 65, 127, 128, 129, 200]
@@ -209,7 +216,7 @@ def test_latent_attention_finds_one_far_key(dtype, far):
     """The last row's query is made to fit one key hundreds of tokens back (the first key, keys on both sides of page and
     tile borders): its result is that key's values, which a key lost or shifted by one would not give."""
     n = 700
-    got, want = _latent_case(5 + far, 2, 16, 4, 12, 24, 4, None, [n - 2, n - 1], 16, dtype, sharp=(n - 1, far))
+    got, want = _latent_case(5 + far, 2, 16, 32, 12, 32, 4, None, [n - 2, n - 1], 16, dtype, sharp=(n - 1, far))
     close(got, want, 1e-4 if dtype == torch.float32 else 3e-2)
 
 
