@@ -1,6 +1,9 @@
 // Latent attention on the matrix cores (bfloat16): the attention of latent.hip for steps whose sizes the 16x16x32
 // instruction takes (latent C a multiple of 16 up to 512, C + R a multiple of 32, pages of a multiple of 8 tokens).
 //
+// Decoded rows (one row of a request in the step) share out their context: blocks of 128 keys each go to an item of their
+// own, which stores partial sums, and a second kernel joins them (so a decoded row's bits depend on its own context
+// only, never on the batch; against the same row inside a prompt portion they differ by rounding).
 // An item is one wave and up to 16 columns; a column is a (row, head) pair: the heads head0 .. head0 + heads - 1 of the rows
 // row0 .. row0 + rows - 1 of one request (rows * heads <= 16).  All heads read the same cached rows, so one key tile serves
 // all 16 columns.  The item walks the request's keys in segments of 64 absolute positions up to its last row's position:
@@ -26,33 +29,53 @@ struct LatentMfmaArgs {
     const int* pos;
     const int* row_entry;
     const int* tables;
-    const int* items;       // [n_items, 4]: row0, rows, head0, heads
+    const int* items;       // [n_items, 8]: row0, rows, head0, heads, key_begin, key_end, slot, -
     bf16_t* out;            // [H, T, C]
+    float* part_o;          // [slots, 16, C]: a split item's sums, not yet divided
+    float* part_ml;         // [slots, 16, 2]: its maximum and its sum of weights
     float scale;
     int T, H, C, R, page_tokens, max_blocks;
 };
 
 #define LM_SEG 64
+#define LM_ITEM_INTS 8
+#define LM_KSTEPS 6     // k-steps of 32 dims whose key loads are in flight together
+#define LM_VTILES 16    // dim tiles of 16 whose value loads are in flight together
 
+// An item with slot < 0 walks all keys up to its last row's position and stores the finished rows.  A split item (one
+// decoded row, the keys key_begin .. key_end - 1, a multiple of 64 apart) stores its unnormalized sums, maximum and sum
+// of weights in its slot; the merge kernel joins a column's slots in key order.
 template <int CT>
 __global__ void __launch_bounds__(64) latent_attention_mfma_kernel(LatentMfmaArgs a) {
     extern __shared__ __align__(16) bf16_t qs[];   // [16][C + R + 8]
     const int lane = threadIdx.x, col = lane & 15, g = lane >> 4;
-    const int* item = a.items + 4 * (size_t)blockIdx.x;
-    const int row0 = item[0], rows = item[1], head0 = item[2], heads = item[3];
+    const int* item = a.items + LM_ITEM_INTS * (size_t)blockIdx.x;
+    const int row0 = item[0], rows = item[1], head0 = item[2], heads = item[3], slot = item[6];
     const int C = a.C, R = a.R, CR = C + R, ldq = CR + 8, pt = a.page_tokens;
     const int n_cols = rows * heads;
 
-    // the columns' queries into LDS, 16 bytes a lane and turn; columns without a (row, head) hold zeros
-    for (int c = 0; c < 16; ++c) {
-        const bool in = c < n_cols;
-        const int r = row0 + (in ? c / heads : 0), h = head0 + (in ? c % heads : 0);
-        const bf16_t* ql = a.q_lat + ((size_t)h * a.T + r) * C;
-        const bf16_t* qr = a.q_rot + ((size_t)h * a.T + r) * R;
-        for (int d = 8 * lane; d < CR; d += 8 * 64) {
-            uint4 v = uint4{0, 0, 0, 0};
-            if (in) v = d < C ? *reinterpret_cast<const uint4*>(ql + d) : *reinterpret_cast<const uint4*>(qr + (d - C));
-            *reinterpret_cast<uint4*>(qs + c * ldq + d) = v;
+    // the columns' queries into LDS, 16 bytes a lane and turn, eight turns' loads in flight together; columns without a
+    // (row, head) hold zeros
+    {
+        const int per_col = CR / 8, chunks = 16 * per_col;
+        for (int i0 = lane; i0 < chunks; i0 += 64 * 8) {
+            uint4 v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const int i = i0 + 64 * u;
+                const int c = i / per_col, d = 8 * (i % per_col);
+                v[u] = uint4{0, 0, 0, 0};
+                if (i < chunks && c < n_cols) {
+                    const int r = row0 + c / heads, h = head0 + c % heads;
+                    v[u] = d < C ? *reinterpret_cast<const uint4*>(a.q_lat + ((size_t)h * a.T + r) * C + d)
+                                 : *reinterpret_cast<const uint4*>(a.q_rot + ((size_t)h * a.T + r) * R + (d - C));
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const int i = i0 + 64 * u;
+                if (i < chunks) *reinterpret_cast<uint4*>(qs + (i / per_col) * ldq + 8 * (i % per_col)) = v[u];
+            }
         }
     }
     __syncthreads();
@@ -64,13 +87,15 @@ __global__ void __launch_bounds__(64) latent_attention_mfma_kernel(LatentMfmaArg
     const int* table = a.tables + (size_t)a.row_entry[row0] * a.max_blocks;
     const int steps = CR / 32;
     const int last_group = (p_max / 8) * 8;
+    const int key_begin = slot < 0 ? 0 : item[4];
+    const int key_last = slot < 0 ? p_max : min(item[5] - 1, p_max);
 
     f32x4_t o[CT];
 #pragma unroll
     for (int dt = 0; dt < CT; ++dt) o[dt] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
     float m = -INFINITY, l = 0.0f;
 
-    for (int seg0 = 0; seg0 <= p_max; seg0 += LM_SEG) {
+    for (int seg0 = key_begin; seg0 <= key_last; seg0 += LM_SEG) {
         // this lane's key row of each of the segment's four score tiles (tile v = 2 * chunk + u)
         const bf16_t* kp[4];
 #pragma unroll
@@ -82,13 +107,27 @@ __global__ void __launch_bounds__(64) latent_attention_mfma_kernel(LatentMfmaArg
         f32x4_t s[4];
 #pragma unroll
         for (int v = 0; v < 4; ++v) s[v] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
-        for (int st = 0; st < steps; ++st) {
-            const bf16x8_t qf = *reinterpret_cast<const bf16x8_t*>(qs + col * ldq + 32 * st + 8 * g);
-            bf16x8_t kf[4];
+        for (int st0 = 0; st0 < steps; st0 += LM_KSTEPS) {
+            // every load of the group is asked for before the first product; a step past the end reads the last step's keys
+            // again and multiplies them by zeros
+            bf16x8_t kf[LM_KSTEPS][4], qf[LM_KSTEPS];
 #pragma unroll
-            for (int v = 0; v < 4; ++v) kf[v] = *reinterpret_cast<const bf16x8_t*>(kp[v] + 32 * st);
+            for (int j = 0; j < LM_KSTEPS; ++j) {
+                const int st = st0 + j < steps ? st0 + j : steps - 1;
 #pragma unroll
-            for (int v = 0; v < 4; ++v) s[v] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[v], qf, s[v], 0, 0, 0);
+                for (int v = 0; v < 4; ++v) kf[j][v] = *reinterpret_cast<const bf16x8_t*>(kp[v] + 32 * st);
+            }
+#pragma unroll
+            for (int j = 0; j < LM_KSTEPS; ++j) {
+                const int st = st0 + j < steps ? st0 + j : steps - 1;
+                const uint4 q = *reinterpret_cast<const uint4*>(qs + col * ldq + 32 * st + 8 * g);
+                const uint4 used = st0 + j < steps ? q : uint4{0, 0, 0, 0};
+                qf[j] = __builtin_bit_cast(bf16x8_t, used);
+            }
+#pragma unroll
+            for (int j = 0; j < LM_KSTEPS; ++j)
+#pragma unroll
+                for (int v = 0; v < 4; ++v) s[v] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[j][v], qf[j], s[v], 0, 0, 0);
         }
         // s[v][i]: key seg0 + 32 (v / 2) + 8 g + 4 (v % 2) + i against column `col`
         float top = -INFINITY;
@@ -101,7 +140,7 @@ __global__ void __launch_bounds__(64) latent_attention_mfma_kernel(LatentMfmaArg
                 top = fmaxf(top, s[v][i]);
             }
         top = rows_max4(top);
-        const float m_new = fmaxf(m, top);           // finite from the first segment on: key 0 counts for every column
+        const float m_new = fmaxf(m, top);           // finite from the first segment on: its first key counts for every column
         const float correction = __expf(m - m_new);  // 0 in the first segment, 1 where the segment holds no key of the column
         float sum = 0.0f;
         bf16x8_t pf[2];
@@ -123,13 +162,29 @@ __global__ void __launch_bounds__(64) latent_attention_mfma_kernel(LatentMfmaArg
             key0 = key0 < last_group ? key0 : last_group;   // a group wholly beyond the last key weighs nothing; read one that exists
             const bf16_t* vp = a.cache_t + ((size_t)table[key0 / pt] * C + col) * pt + key0 % pt;
 #pragma unroll
-            for (int dt = 0; dt < CT; ++dt) {
-                if (16 * dt < C) {
-                    const bf16x8_t vf = *reinterpret_cast<const bf16x8_t*>(vp + (size_t)16 * dt * pt);
-                    o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[c], o[dt], 0, 0, 0);
+            for (int d0 = 0; d0 < CT; d0 += LM_VTILES) {
+                bf16x8_t vf[LM_VTILES < CT ? LM_VTILES : CT];
+#pragma unroll
+                for (int j = 0; j < (LM_VTILES < CT ? LM_VTILES : CT); ++j) {
+                    const int dt = 16 * (d0 + j) < C ? d0 + j : 0;     // a tile past the latent reads the first one again; its product is dropped
+                    vf[j] = *reinterpret_cast<const bf16x8_t*>(vp + (size_t)16 * dt * pt);
                 }
+#pragma unroll
+                for (int j = 0; j < (LM_VTILES < CT ? LM_VTILES : CT); ++j)
+                    if (16 * (d0 + j) < C) o[d0 + j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[j], pf[c], o[d0 + j], 0, 0, 0);
             }
         }
+    }
+    if (slot >= 0) {
+        float* po = a.part_o + ((size_t)slot * 16 + col) * C;
+#pragma unroll
+        for (int dt = 0; dt < CT; ++dt)
+            if (16 * dt < C) *reinterpret_cast<f32x4_t*>(po + 16 * dt + 4 * g) = o[dt];
+        if (g == 0) {
+            a.part_ml[((size_t)slot * 16 + col) * 2] = m;
+            a.part_ml[((size_t)slot * 16 + col) * 2 + 1] = l;
+        }
+        return;
     }
     if (!live) return;
     bf16_t* out = a.out + ((size_t)c_head * a.T + c_row) * C;
@@ -143,23 +198,80 @@ __global__ void __launch_bounds__(64) latent_attention_mfma_kernel(LatentMfmaArg
     }
 }
 
+// Joins the slots of a decoded row's split items, in key order: with M the largest of the slots' maxima,
+// out = sum_i O_i e^(m_i - M) / sum_i l_i e^(m_i - M).  merges [n, 8]: row, head0, heads, first slot, slots.
+// One workgroup a column (blockIdx.y): the slots' weights are formed once into LDS, then every thread adds its dims over
+// the slots in order, eight slots' loads in flight.
+#define LM_MERGE_MAX 1024    // slots of one column whose weights fit the workgroup's LDS; longer columns take rounds
+__global__ void __launch_bounds__(256) latent_attention_merge_kernel(const int* __restrict__ merges, const float* __restrict__ part_o,
+                                                                   const float* __restrict__ part_ml, bf16_t* __restrict__ out, int T, int C) {
+    __shared__ float weight[LM_MERGE_MAX];
+    __shared__ float scratch[4];
+    const int* mg = merges + LM_ITEM_INTS * (size_t)blockIdx.x;
+    const int row = mg[0], head0 = mg[1], heads = mg[2], slot0 = mg[3], n = mg[4];
+    const int c = blockIdx.y;
+    if (c >= heads) return;
+    // M: every thread takes slots tid, tid + 256, ...; the workgroup's maximum does not depend on the order
+    float M = -INFINITY;
+    for (int i = threadIdx.x; i < n; i += 256) M = fmaxf(M, part_ml[((size_t)(slot0 + i) * 16 + c) * 2]);
+    M = wave_max(M);
+    if ((threadIdx.x & 63) == 0) scratch[threadIdx.x >> 6] = M;
+    __syncthreads();
+    M = fmaxf(fmaxf(scratch[0], scratch[1]), fmaxf(scratch[2], scratch[3]));
+    float acc[2] = {0.0f, 0.0f};    // dims tid and tid + 256 (C <= 512)
+    float L = 0.0f;
+    for (int i0 = 0; i0 < n; i0 += LM_MERGE_MAX) {
+        const int round = min(LM_MERGE_MAX, n - i0);
+        __syncthreads();
+        for (int i = threadIdx.x; i < round; i += 256) weight[i] = __expf(part_ml[((size_t)(slot0 + i0 + i) * 16 + c) * 2] - M);
+        __syncthreads();
+        for (int i = 0; i < round; ++i) L += part_ml[((size_t)(slot0 + i0 + i) * 16 + c) * 2 + 1] * weight[i];   // in slot order, by every thread alike
+        for (int i = 0; i < round; i += 8) {
+            float v[8][2];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const int at = i + u < round ? i + u : round - 1;
+                const float* po = part_o + ((size_t)(slot0 + i0 + at) * 16 + c) * C;
+#pragma unroll
+                for (int e = 0; e < 2; ++e) v[u][e] = threadIdx.x + 256 * e < C ? po[threadIdx.x + 256 * e] : 0.0f;
+            }
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+                if (i + u < round) {
+                    acc[0] += v[u][0] * weight[i + u];
+                    acc[1] += v[u][1] * weight[i + u];
+                }
+        }
+    }
+    const float inv = 1.0f / L;
+#pragma unroll
+    for (int e = 0; e < 2; ++e)
+        if (threadIdx.x + 256 * e < C) out[((size_t)(head0 + c) * T + row) * C + threadIdx.x + 256 * e] = f32_to_bf16(acc[e] * inv);
+}
+
 extern "C" int llmx_latent_attention_mfma_ok(int C, int R, int page_tokens) {
     return C >= 16 && C <= 512 && C % 16 == 0 && R >= 0 && R % 8 == 0 && (C + R) % 32 == 0 && page_tokens > 0 && page_tokens % 8 == 0 ? 1 : 0;
 }
 
 extern "C" int llmx_latent_attention_mfma(const void* q_lat, const void* q_rot, const void* cache, const void* cache_t, const int* pos,
-                                          const int* row_entry, const int* tables, const int* items, int n_items, void* out, float scale, int T,
-                                          int H, int C, int R, int page_tokens, int max_blocks, hipStream_t stream) {
+                                          const int* row_entry, const int* tables, const int* items, int n_items, const int* merges, int n_merges,
+                                          void* out, float* part_o, float* part_ml, float scale, int T, int H, int C, int R, int page_tokens,
+                                          int max_blocks, hipStream_t stream) {
     if (n_items <= 0) return 0;
     if (!llmx_latent_attention_mfma_ok(C, R, page_tokens)) return -2;
     llmx_note_launch(LK_LATENT_ATTENTION_MFMA);
+    if (n_merges > 0 && (!merges || !part_o || !part_ml)) return -2;
     LatentMfmaArgs a{(const bf16_t*)q_lat, (const bf16_t*)q_rot, (const bf16_t*)cache, (const bf16_t*)cache_t, pos, row_entry, tables, items,
-                     (bf16_t*)out, scale, T, H, C, R, page_tokens, max_blocks};
+                     (bf16_t*)out, part_o, part_ml, scale, T, H, C, R, page_tokens, max_blocks};
     const size_t lds = sizeof(bf16_t) * 16 * (size_t)(C + R + 8);
     const dim3 grid(n_items), block(64);
     if (C <= 64) hipLaunchKernelGGL(latent_attention_mfma_kernel<4>, grid, block, lds, stream, a);
     else if (C <= 128) hipLaunchKernelGGL(latent_attention_mfma_kernel<8>, grid, block, lds, stream, a);
     else if (C <= 256) hipLaunchKernelGGL(latent_attention_mfma_kernel<16>, grid, block, lds, stream, a);
     else hipLaunchKernelGGL(latent_attention_mfma_kernel<32>, grid, block, lds, stream, a);
+    if (n_merges > 0) {
+        llmx_note_launch(LK_LATENT_ATTENTION_MERGE);
+        hipLaunchKernelGGL(latent_attention_merge_kernel, dim3(n_merges, 16), dim3(256), 0, stream, merges, part_o, part_ml, (bf16_t*)out, T, C);
+    }
     return LLMX_CHECK_LAUNCH();
 }

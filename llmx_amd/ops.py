@@ -60,8 +60,9 @@ def _declare(h) -> None:
         "llmx_act_xielu": [P, P, P, I, L, P],
         "llmx_act_gelu_gather": [P, P, I, P, P, I, I, I, I, I, P],
         "llmx_mingru_scan": [P, P, P, P, P, P, P, P, I, I, I, P],
+        "llmx_mingru_scan_chunks": [P, P, P, P, P, P, P, P, I, I, I, P, I, P, P, P, P],
         "llmx_latent_prep": [P, P, P, P, P, P, P, P, P, P, I, F, I, I, I, I, I, I, I, I, I, I, P],
-        "llmx_latent_attention_mfma": [P, P, P, P, P, P, P, P, I, P, F, I, I, I, I, I, I, P],
+        "llmx_latent_attention_mfma": [P, P, P, P, P, P, P, P, I, P, I, P, P, P, F, I, I, I, I, I, I, P],
         "llmx_latent_attention_mfma_ok": [I, I, I],
         "llmx_latent_attention_generic": [P, P, P, P, P, P, P, I, F, I, I, I, I, I, I, I, P],
         "llmx_head_gate": [P, P, I, P, I, I, I, I, P],
@@ -224,16 +225,68 @@ def act_gelu_gather(z: torch.Tensor, table: torch.Tensor, ids: torch.Tensor, out
            "act_gelu_gather")
 
 
+SCAN_CHUNK_ROWS = 64         # rows of a chunk of the recurrence's three-launch form
+SCAN_CHUNKS_MIN_ROWS = 256   # an entry of at least this many rows in the step: the three-launch form runs
+
+
+class ScanPlan:
+    """The chunks of a step's rows for the recurrence's three-launch form (it holds no positions and no slots)."""
+
+    def __init__(self, row_counts, device):
+        import numpy as np
+        chunks, per_entry, row0 = [], [], 0
+        for e, n in enumerate(row_counts):
+            first = len(chunks)
+            for r in range(0, n, SCAN_CHUNK_ROWS):
+                chunks.append([e, row0 + r, min(SCAN_CHUNK_ROWS, n - r), 1 if r + SCAN_CHUNK_ROWS >= n else 0])
+            per_entry.append([first, len(chunks) - first])
+            row0 += n
+        self.n_chunks = len(chunks)
+        self.chunks = torch.tensor(np.asarray(chunks, dtype=np.int32), device=device)
+        self.entry_chunks = torch.tensor(np.asarray(per_entry, dtype=np.int32), device=device)
+
+
+_SCAN_PLANS: dict = {}
+
+
+def scan_plan(row_counts, device) -> Optional[ScanPlan]:
+    """The chunk lists for a step with these rows an entry, or None when no entry is long enough for them to pay."""
+    if max(row_counts) < SCAN_CHUNKS_MIN_ROWS:
+        return None
+    key = (tuple(row_counts), str(device))
+    plan = _SCAN_PLANS.get(key)
+    if plan is None:
+        if len(_SCAN_PLANS) > 64:
+            _SCAN_PLANS.clear()
+        plan = _SCAN_PLANS[key] = ScanPlan(row_counts, device)
+    return plan
+
+
 def mingru_scan(zxg: torch.Tensor, bz: Optional[torch.Tensor], bx: Optional[torch.Tensor], state: torch.Tensor, slot_read: torch.Tensor,
-                slot_write: torch.Tensor, entry_rows: torch.Tensor, out: torch.Tensor) -> None:
+                slot_write: torch.Tensor, entry_rows: torch.Tensor, out: torch.Tensor, plan: Optional[ScanPlan] = None, scratch=None) -> None:
     """The minGRU recurrence over each entry's rows (see csrc/recurrent.hip): zxg [T, 3W] float32 pre-activations
     (gate | candidate | output gate), state [slots, W] float32 read at slot_read[e] and written at slot_write[e],
-    entry_rows [n_entries, 2] (first row, rows); out [T, W] = S_t * silu(g_t)."""
+    entry_rows [n_entries, 2] (first row, rows); out [T, W] = S_t * silu(g_t).  With a `plan` (scan_plan) the rows are
+    worked on in chunks by three launches; `scratch(name, shape, dtype)` gives them storage."""
     T, W3 = zxg.shape
     W = W3 // 3
     n_e = entry_rows.shape[0]
     if W3 != 3 * W or state.shape[1] != W or tuple(out.shape) != (T, W):
         raise KernelError("mingru_scan: shapes do not agree")
+    if plan is not None:
+        if plan.entry_chunks.shape[0] != n_e:
+            raise KernelError("mingru_scan: the plan does not fit the step's entries")
+        if scratch is None:
+            scratch = lambda name, shape, dtype: torch.empty(shape, dtype=dtype, device=zxg.device)
+        chunk_a = scratch("scan.chunk_a", (plan.n_chunks, W), torch.float32)
+        chunk_b = scratch("scan.chunk_b", (plan.n_chunks, W), torch.float32)
+        _check(lib().llmx_mingru_scan_chunks(_dev(zxg, "zxg", torch.float32), _dev(bz, "bz", torch.float32, (W,)), _dev(bx, "bx", torch.float32, (W,)),
+                                             _dev(state, "state", torch.float32), _dev(slot_read, "slot_read", torch.int32, (n_e,)),
+                                             _dev(slot_write, "slot_write", torch.int32, (n_e,)), _dev(entry_rows, "entry_rows", torch.int32, (n_e, 2)),
+                                             _dev(out, "out"), _code(out.dtype), n_e, W, _dev(plan.chunks, "chunks", torch.int32, (plan.n_chunks, 4)),
+                                             plan.n_chunks, _dev(plan.entry_chunks, "entry_chunks", torch.int32, (n_e, 2)),
+                                             _dev(chunk_a, "chunk_a"), _dev(chunk_b, "chunk_b"), _stream()), "mingru_scan_chunks")
+        return
     _check(lib().llmx_mingru_scan(_dev(zxg, "zxg", torch.float32), _dev(bz, "bz", torch.float32, (W,)), _dev(bx, "bx", torch.float32, (W,)),
                                   _dev(state, "state", torch.float32), _dev(slot_read, "slot_read", torch.int32, (n_e,)),
                                   _dev(slot_write, "slot_write", torch.int32, (n_e,)), _dev(entry_rows, "entry_rows", torch.int32, (n_e, 2)),
@@ -278,10 +331,18 @@ def latent_attention(q_lat: torch.Tensor, q_rot: torch.Tensor, cache: torch.Tens
     if cache_t is not None and plan is not None and window == 0 and latent_attention_mfma_ok(q_lat.dtype, C, R, page_tokens):
         if plan.heads != H or plan.rows != T or tuple(cache_t.shape) != (n_pages, C, page_tokens) or cache_t.dtype != cache.dtype:
             raise KernelError("latent_attention: the plan or the transposed copy does not fit the step")
+        part_o = part_ml = None
+        if plan.n_slots:
+            if scratch is None:
+                scratch = lambda name, shape, dtype: torch.empty(shape, dtype=dtype, device=q_lat.device)
+            part_o = scratch("latent.part_o", (plan.n_slots, 16, C), torch.float32)
+            part_ml = scratch("latent.part_ml", (plan.n_slots, 16, 2), torch.float32)
         _check(lib().llmx_latent_attention_mfma(_dev(q_lat, "q_lat"), _dev(q_rot, "q_rot"), _dev(cache, "cache"), _dev(cache_t, "cache_t"),
                                                 _dev(pos, "pos", torch.int32, (T,)), _dev(row_entry, "row_entry", torch.int32, (T,)),
                                                 _dev(tables, "tables", torch.int32), _dev(plan.items, "items", torch.int32), plan.n_items,
-                                                _dev(out, "out"), float(scale), T, H, C, R, page_tokens, tables.shape[1], _stream()),
+                                                _dev(plan.merges, "merges", torch.int32), plan.n_merges, _dev(out, "out"),
+                                                _dev(part_o, "part_o"), _dev(part_ml, "part_ml"), float(scale), T, H, C, R, page_tokens,
+                                                tables.shape[1], _stream()),
                "latent_attention_mfma")
         return
     _check(lib().llmx_latent_attention_generic(_dev(q_lat, "q_lat"), _dev(q_rot, "q_rot"), _dev(cache, "cache"), _dev(pos, "pos", torch.int32, (T,)),
@@ -294,36 +355,51 @@ def latent_attention_mfma_ok(dtype: torch.dtype, rank: int, rot_dim: int, page_t
     return dtype == torch.bfloat16 and bool(lib().llmx_latent_attention_mfma_ok(int(rank), int(rot_dim), int(page_tokens)))
 
 
-class LatentPlan:
-    """Work items of the matrix-core latent attention for one step's rows: each up to 16 (row, head) columns of one request.
-    It holds no positions, so one plan serves every step with the same rows a request."""
+LATENT_SPLIT_KEYS = 128    # keys a split item of a decoded row takes (two segments of the kernel)
 
-    def __init__(self, items, heads, rows, device):
+
+class LatentPlan:
+    """Work items of the matrix-core latent attention for one step's rows: each up to 16 (row, head) columns of one request,
+    whole or, for decoded rows, one block of the context; and the list of joins of the split ones.  It holds no positions."""
+
+    def __init__(self, items, merges, n_slots, heads, rows, device):
         import numpy as np
-        self.heads, self.rows, self.n_items = heads, rows, len(items)
-        self.items = torch.tensor(np.asarray(items, dtype=np.int32).reshape(-1, 4), device=device)
+        self.heads, self.rows, self.n_items, self.n_merges, self.n_slots = heads, rows, len(items), len(merges), n_slots
+        self.items = torch.tensor(np.asarray(items, dtype=np.int32).reshape(-1, 8), device=device)
+        self.merges = torch.tensor(np.asarray(merges, dtype=np.int32).reshape(-1, 8), device=device) if merges else None
 
 
 _LATENT_PLANS: dict = {}
 
 
-def latent_plan(row_counts, heads: int, device) -> LatentPlan:
-    """row_counts[i]: rows of entry i (entries' rows are consecutive, in order).  With 16 heads or more an item is one row and
-    up to 16 of its heads; with fewer, 16 // heads consecutive rows of one entry with all their heads.  Later rows (longer
-    key ranges) come first."""
-    key = (tuple(row_counts), heads, str(device))
+def latent_plan(row_counts, heads: int, device, contexts=None) -> LatentPlan:
+    """row_counts[i]: rows of entry i (entries' rows are consecutive, in order); contexts[i]: the tokens it holds after the
+    step (None: nothing is split).  With 16 heads or more an item is one row and up to 16 of its heads; with fewer,
+    16 // heads consecutive rows of one entry with all their heads; later rows (longer key ranges) come first.  An entry of
+    one row (a decoded token) whose context is longer than LATENT_SPLIT_KEYS gets an item for every block of that many
+    keys, a function of its own context only."""
+    blocks = tuple(-(-c // LATENT_SPLIT_KEYS) if n == 1 else 1 for n, c in zip(row_counts, contexts)) if contexts is not None else None
+    key = (tuple(row_counts), heads, blocks, str(device))
     plan = _LATENT_PLANS.get(key)
     if plan is None:
-        items, row0 = [], 0
+        items, merges, row0, slot = [], [], 0, 0
         per = max(1, 16 // heads)
-        for n in row_counts:
+        for i, n in enumerate(row_counts):
+            nb = blocks[i] if blocks is not None else 1
             for r in range(((n - 1) // per) * per, -1, -per):
                 for h0 in range(0, heads, 16):
-                    items.append([row0 + r, min(per, n - r), h0, min(16, heads - h0)])
+                    nh = min(16, heads - h0)
+                    if nb <= 1:
+                        items.append([row0 + r, min(per, n - r), h0, nh, 0, 0, -1, 0])
+                        continue
+                    merges.append([row0, h0, nh, slot, nb, 0, 0, 0])
+                    for b in range(nb):
+                        items.append([row0, 1, h0, nh, b * LATENT_SPLIT_KEYS, (b + 1) * LATENT_SPLIT_KEYS, slot + b, 0])
+                    slot += nb
             row0 += n
         if len(_LATENT_PLANS) > 256:
             _LATENT_PLANS.clear()
-        plan = _LATENT_PLANS[key] = LatentPlan(items, heads, row0, device)
+        plan = _LATENT_PLANS[key] = LatentPlan(items, merges, slot, heads, row0, device)
     return plan
 
 

@@ -100,7 +100,8 @@ class LatentAttention(Mixer):
     def _plan(self, step):
         if not self._matrix_cores():
             return None
-        return step.shared(("latent.plan", self.heads), lambda: ops.latent_plan([e.n for e in step.entries], self.heads, step.device))
+        return step.shared(("latent.plan", self.heads), lambda: ops.latent_plan([e.n for e in step.entries], self.heads, step.device,
+                                                                                 contexts=[e.past + e.n for e in step.entries]))
 
     def graph_key(self, step):
         # a recorded step reads the groups' lists and the plan's items; the key keeps them alive

@@ -53,7 +53,10 @@ class MinGRU(Mixer):
         pre = step.buf("mingru.pre", (T, 3 * W), torch.float32)
         ops.gemm(h, self.w_in, pre, scratch=step.buf)
         gated = step.buf("mingru.gated", (T, W), step.act_dtype)
-        ops.mingru_scan(pre, self.b_z, self.b_x, cache.state, step.entry_held_slots, step.entry_slots, step.entry_rows, gated)
+        # long runs of rows (a prompt's portion) are worked on in chunks; a decode step's entries never are (nothing for a graph to hold)
+        plan = step.shared("scan.plan", lambda: ops.scan_plan([e.n for e in step.entries], step.device))
+        ops.mingru_scan(pre, self.b_z, self.b_x, cache.state, step.entry_held_slots, step.entry_slots, step.entry_rows, gated,
+                        plan=plan, scratch=step.buf)
         ops.gemm(gated, self.w_o, out, ops.EPI_ADD if accumulate else ops.EPI_STORE, scratch=step.buf)
 
 

@@ -23,6 +23,7 @@ pytestmark = pytest.mark.gpu
 
 F32_TOL = 2e-5      # |engine - plain| over all logits relative to the largest |logit|, float32 sums in another order
 BF16_TOL = 2.5e-2   # both round at the same places; single bfloat16 roundings flip on last-bit differences of the sums
+CUT_TOL = 1.5e-2    # bfloat16, one cutting against another: see same_rows
 
 
 def ops():
@@ -134,6 +135,41 @@ def test_gated_recurrence_rows_state_and_slots(W):
     assert float(state[7].min()) == 7.0 and float(state[4].max()) == 7.0      # slots of no request are untouched
 
 
+def test_gated_recurrence_in_chunks():
+    """Long runs of rows take the three-launch form (chunks of 64 rows): two requests of 700 and 3 rows beside one of 257,
+    from given states, against the plain recurrence and against the one-launch form."""
+    g = torch.Generator().manual_seed(9)
+    W, E = 70, 16
+    w = {"m.z": torch.randn(W, E, generator=g), "m.x": torch.randn(W, E, generator=g) * 2, "m.g": torch.randn(W, E, generator=g),
+         "m.z.b": torch.randn(W, generator=g), "m.x.b": torch.randn(W, generator=g), "m.o": torch.eye(W)}
+    lengths = [700, 3, 257]
+    hs = [torch.randn(n, E, generator=g) for n in lengths]
+    starts = torch.rand(3, W, generator=g)
+    want = [plain.mingru(h.double(), w, "m.", {"width": W}, state=starts[i].double()) for i, h in enumerate(hs)]
+    pre = dev(torch.cat(hs) @ torch.cat([w["m.z"], w["m.x"], w["m.g"]]).T)
+    rows = dev(torch.tensor([[0, 700], [700, 3], [703, 257]], dtype=torch.int32))
+    reads, writes = dev(torch.tensor([0, 1, 2], dtype=torch.int32)), dev(torch.tensor([5, 4, 3], dtype=torch.int32))
+    outs = []
+    for chunked in (True, False):
+        state = torch.zeros(6, W, device="cuda")
+        state[:3] = dev(starts)
+        out = torch.empty(960, W, dtype=torch.float32, device="cuda")
+        plan = ops().scan_plan(lengths, "cuda") if chunked else None
+        assert (plan is not None) == chunked
+        ops().take_launches()
+        ops().mingru_scan(pre, dev(w["m.z.b"]), dev(w["m.x.b"]), state, reads, writes, rows, out, plan=plan)
+        assert ("gated_scan.chunks" in ops().take_launches()) == chunked
+        at = 0
+        for i, n in enumerate(lengths):
+            close(out[at:at + n], want[i][0], 2e-5)
+            close(state[5 - i], want[i][1], 2e-5)
+            at += n
+        assert torch.equal(state[:3].cpu(), starts)
+        outs.append(out)
+    close(outs[0], outs[1], 1e-5)
+    assert ops().scan_plan([255, 1, 30], "cuda") is None
+
+
 def _latent_case(seed, H, D, R, V, C, dims, scaling, positions, page, dtype, sharp=None):
     """One latent-attention layer on the kernels (products by torch) for rows at `positions` of one request whose earlier
     tokens are already cached in shuffled pages, against plain.latent_attention over the whole sequence."""
@@ -189,8 +225,10 @@ def _latent_case(seed, H, D, R, V, C, dims, scaling, positions, page, dtype, sha
         mixed = torch.empty(H, T, C, dtype=dtype, device="cuda")
         o.take_launches()
         o.latent_attention(q_lat, q_rot, cache, pos, entry, tables, mixed, 0.3, cache_t=cache_t,
-                           plan=o.latent_plan([0, T], H, "cuda") if cores else None)
-        assert ("latent_attention.mfma" in o.take_launches()) == cores
+                           plan=o.latent_plan([0, T], H, "cuda", contexts=[0, max(rows) + 1]) if cores else None)
+        ran = o.take_launches()
+        assert ("latent_attention.mfma" in ran) == cores
+        assert ("latent_attention.merge" in ran) == (cores and T == 1 and max(rows) >= o.LATENT_SPLIT_KEYS)
         values = torch.bmm(mixed.float(), uv.float().transpose(1, 2)).contiguous()
         joined = torch.empty(T, H * V, dtype=dtype, device="cuda")
         o.head_gate(values, proj[:, H * (D + R) + C + R:], joined)
@@ -218,6 +256,9 @@ def test_latent_attention_finds_one_far_key(dtype, far):
     n = 700
     got, want = _latent_case(5 + far, 2, 16, 32, 12, 32, 4, None, [n - 2, n - 1], 16, dtype, sharp=(n - 1, far))
     close(got, want, 1e-4 if dtype == torch.float32 else 3e-2)
+    # the same row decoded alone: in bfloat16 its context is shared out over work items and joined
+    got, want = _latent_case(5 + far, 2, 16, 32, 12, 32, 4, None, [n - 1], 16, dtype, sharp=(n - 1, far))
+    close(got, want, 1e-4 if dtype == torch.float32 else 3e-2)
 
 
 # ---------------------------------------------------------------------------
@@ -239,6 +280,16 @@ def run_cut(engine, rid, tokens, cuts):
     rows = [engine.step([StepEntry(rid, tokens[a:b], list(range(b - a)))]).clone() for a, b in cuts]
     engine.end_request(rid)
     return torch.cat(rows).cpu()
+
+
+def same_rows(got, whole, dtype, what, tol=CUT_TOL):
+    """Two cuttings of the same tokens.  float32: the same bits.  bfloat16: the same bits except that a token decoded alone
+    shares out its context over work items of the matrix-core latent attention, whose partial sums are joined in another
+    order than a prompt portion's row walks its keys: such rows agree within rounding."""
+    if dtype == "float32":
+        assert torch.equal(got, whole), f"{what}: rows differ, first at row {int((got != whole).any(1).nonzero()[0])}"
+    else:
+        close(got, whole, tol)
 
 
 def against_plain(name, dtype, length, seed, got):
@@ -272,8 +323,8 @@ def test_whole_prompts_and_every_layer(setup):
 
 
 def test_prompt_against_token_by_token_and_portions(setup):
-    """Every cutting gives every row the same bits: whole, token by token from the first token, most of it whole and the
-    rest one by one, and portions of changing size down to two tokens and to one."""
+    """Every cutting gives every row the same values: whole, token by token from the first token, most of it whole and the
+    rest one by one, and portions of changing size down to two tokens and to one (same_rows says what "the same" is)."""
     name, dtype, engine = setup
     length, seed = 130, 5
     tokens = tokens_for(name, length, seed)
@@ -287,14 +338,15 @@ def test_prompt_against_token_by_token_and_portions(setup):
         "pairs": [(i, min(i + 2, length)) for i in range(0, length, 2)],
     }
     for what, cuts in cuttings.items():
-        got = run_cut(engine, what, tokens, cuts)
-        assert torch.equal(got, whole), f"{what}: rows differ from the whole prompt's, first at row {int((got != whole).any(1).nonzero()[0])}"
+        same_rows(run_cut(engine, what, tokens, cuts), whole, dtype, what)
+    # portions of at least two tokens walk their keys as the whole prompt does: the same bits in bfloat16 too
+    assert torch.equal(run_cut(engine, "pairs", tokens, cuttings["pairs"]), whole)
 
 
 def test_unequal_requests_in_one_batch_and_reused_pages_and_slots(setup):
     """Four requests of unequal length advance together, portions of some beside single tokens of others, in an engine
     with four seats and so few pages that ended requests' pages and slots are taken again by later ones; every row has
-    the bits it has when its request runs alone in a fresh engine."""
+    the bits it has when its request runs alone, cut the same way, in a fresh engine, and the whole prompt's rows."""
     from llmx_amd.engine import StepEntry
     name, dtype, _ = setup
     lengths = [70, 23, 1, 96, 40, 17, 64, 5]
@@ -303,7 +355,7 @@ def test_unequal_requests_in_one_batch_and_reused_pages_and_slots(setup):
     engine = make_engine(name, dtype, kv_tokens=4 * 112, max_requests=4)
     rng = random.Random(3)
     waiting = list(range(len(lengths)))
-    live, fed, got = [], {}, {i: [] for i in range(len(lengths))}
+    live, fed, got, cuts = [], {}, {i: [] for i in range(len(lengths))}, {i: [] for i in range(len(lengths))}
     while waiting or live:
         while waiting and len(live) < 4:
             i = waiting.pop(0)
@@ -324,13 +376,16 @@ def test_unequal_requests_in_one_batch_and_reused_pages_and_slots(setup):
         at = 0
         for i, n in taken:
             got[i].append(out[at:at + n])
+            cuts[i].append((fed[i], fed[i] + n))
             at += n
             fed[i] += n
             if fed[i] == lengths[i]:
                 engine.end_request(i)
                 live.remove(i)
     for i in range(len(lengths)):
-        assert torch.equal(torch.cat(got[i]), alone[i]), f"request {i} differs from its run alone"
+        same_rows(torch.cat(got[i]), alone[i], dtype, f"request {i} against its whole prompt")
+        again = run_cut(alone_engine, ("again", i), tokens_for(name, lengths[i], 20 + i), cuts[i])
+        assert torch.equal(torch.cat(got[i]), again), f"request {i} differs from its run alone"
     assert engine.cache.pages_in_use(0) == 0 if engine.cache.groups else True
     assert engine.cache.slots.in_use == 0
 
@@ -348,7 +403,20 @@ def test_long_decoding_and_graph_replays(setup):
     against_plain(name, dtype, length, seed, got)
     eager = make_engine(name, dtype, graphs=False)
     assert torch.equal(run_cut(eager, "long", tokens, cuts), got)
-    assert torch.equal(run_cut(eager, "whole", tokens, [(0, length)]), got)
+    same_rows(got, run_cut(eager, "whole", tokens, [(0, length)]), dtype, "decoded against whole")
+
+
+def test_a_long_prompt_in_one_step(setup):
+    """600 tokens in one step: the recurrence runs in chunks and the attention walks many segments; against the plain model,
+    against portions of at most 100 rows (the one-launch recurrence) and against decoding the last 40 tokens."""
+    name, dtype, engine = setup
+    length, seed = 600, 12
+    tokens = tokens_for(name, length, seed)
+    whole = run_cut(engine, "long whole", tokens, [(0, length)])
+    against_plain(name, dtype, length, seed, whole)
+    tol = 2e-5 if dtype == "float32" else CUT_TOL
+    close(run_cut(engine, "long portions", tokens, [(i, min(i + 100, length)) for i in range(0, length, 100)]), whole, tol)
+    close(run_cut(engine, "long decoded", tokens, [(0, 300), (300, length - 40)] + [(i, i + 1) for i in range(length - 40, length)]), whole, tol)
 
 
 def test_a_failed_step_leaves_the_state_as_it_was():
@@ -386,8 +454,9 @@ def test_sharp_attention_over_hundreds_of_tokens(dtype, tmp_path):
     want = plain.forward(cfg, w, tokens, torch.float64, torch.bfloat16 if dtype == "bfloat16" else None)
     whole = run_cut(engine, "w", tokens, [(0, length)])
     close(whole, want, 1e-4 if dtype == "float32" else 6e-2)
-    assert torch.equal(run_cut(engine, "p", tokens, portions(length, 9)), whole)
-    assert torch.equal(run_cut(engine, "d", tokens, [(0, length - 50)] + [(i, i + 1) for i in range(length - 50, length)]), whole)
+    same_rows(run_cut(engine, "p", tokens, portions(length, 9)), whole, dtype, "portions", 6e-2)
+    assert torch.equal(run_cut(engine, "pairs", tokens, [(i, i + 2) for i in range(0, length, 2)]), whole)
+    same_rows(run_cut(engine, "d", tokens, [(0, length - 50)] + [(i, i + 1) for i in range(length - 50, length)]), whole, dtype, "decoded", 6e-2)
 
 
 def test_greedy_generation_through_the_scheduler():
