@@ -59,6 +59,8 @@
     X(LATENT_PREP, "latent_prep")                                                                                         \
     X(LATENT_ATTENTION_GENERIC, "latent_attention.generic")                                                               \
     X(LATENT_ATTENTION_MFMA, "latent_attention.mfma")                                                                     \
+    X(LATENT_ATTENTION_TILES, "latent_attention.tiles")                                                                   \
+    X(LATENT_ATTENTION_ROWS, "latent_attention.rows")                                                                     \
     X(LATENT_ATTENTION_MERGE, "latent_attention.merge")                                                                   \
     X(HEAD_GATE, "head_gate")
 

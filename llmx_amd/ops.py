@@ -62,7 +62,7 @@ def _declare(h) -> None:
         "llmx_mingru_scan": [P, P, P, P, P, P, P, P, I, I, I, P],
         "llmx_mingru_scan_chunks": [P, P, P, P, P, P, P, P, I, I, I, P, I, P, P, P, P],
         "llmx_latent_prep": [P, P, P, P, P, P, P, P, P, P, I, F, I, I, I, I, I, I, I, I, I, I, P],
-        "llmx_latent_attention_mfma": [P, P, P, P, P, P, P, P, I, P, I, P, P, P, F, I, I, I, I, I, I, P],
+        "llmx_latent_attention_mfma": [P, P, P, P, P, P, P, P, I, I, I, P, I, P, P, P, F, I, I, I, I, I, I, P],
         "llmx_latent_attention_mfma_ok": [I, I, I],
         "llmx_latent_attention_generic": [P, P, P, P, P, P, P, I, F, I, I, I, I, I, I, I, P],
         "llmx_head_gate": [P, P, I, P, I, I, I, I, P],
@@ -340,7 +340,7 @@ def latent_attention(q_lat: torch.Tensor, q_rot: torch.Tensor, cache: torch.Tens
         _check(lib().llmx_latent_attention_mfma(_dev(q_lat, "q_lat"), _dev(q_rot, "q_rot"), _dev(cache, "cache"), _dev(cache_t, "cache_t"),
                                                 _dev(pos, "pos", torch.int32, (T,)), _dev(row_entry, "row_entry", torch.int32, (T,)),
                                                 _dev(tables, "tables", torch.int32), _dev(plan.items, "items", torch.int32), plan.n_items,
-                                                _dev(plan.merges, "merges", torch.int32), plan.n_merges, _dev(out, "out"),
+                                                plan.n_tile_items, plan.n_row_items, _dev(plan.merges, "merges", torch.int32), plan.n_merges, _dev(out, "out"),
                                                 _dev(part_o, "part_o"), _dev(part_ml, "part_ml"), float(scale), T, H, C, R, page_tokens,
                                                 tables.shape[1], _stream()),
                "latent_attention_mfma")
@@ -362,9 +362,12 @@ class LatentPlan:
     """Work items of the matrix-core latent attention for one step's rows: each up to 16 (row, head) columns of one request,
     whole or, for decoded rows, one block of the context; and the list of joins of the split ones.  It holds no positions."""
 
-    def __init__(self, items, merges, n_slots, heads, rows, device):
+    def __init__(self, tiles, row_items, items, merges, n_slots, heads, rows, device):
         import numpy as np
         self.heads, self.rows, self.n_items, self.n_merges, self.n_slots = heads, rows, len(items), len(merges), n_slots
+        self.n_tile_items = len(tiles)       # the list's first items: four column tiles each, for a workgroup of four waves
+        self.n_row_items = len(row_items)    # then the decoded rows' items: one column tile, a workgroup of four waves
+        items = tiles + row_items + items
         self.items = torch.tensor(np.asarray(items, dtype=np.int32).reshape(-1, 8), device=device)
         self.merges = torch.tensor(np.asarray(merges, dtype=np.int32).reshape(-1, 8), device=device) if merges else None
 
@@ -372,34 +375,48 @@ class LatentPlan:
 _LATENT_PLANS: dict = {}
 
 
-def latent_plan(row_counts, heads: int, device, contexts=None) -> LatentPlan:
+LATENT_TILES = 4           # column tiles of 16 that a workgroup of the prompt form takes (the kernel's LW_TILES)
+
+
+def latent_plan(row_counts, heads: int, device, contexts=None, tiles: bool = True) -> LatentPlan:
     """row_counts[i]: rows of entry i (entries' rows are consecutive, in order); contexts[i]: the tokens it holds after the
     step (None: nothing is split).  With 16 heads or more an item is one row and up to 16 of its heads; with fewer,
     16 // heads consecutive rows of one entry with all their heads; later rows (longer key ranges) come first.  An entry of
     one row (a decoded token) whose context is longer than LATENT_SPLIT_KEYS gets an item for every block of that many
-    keys, a function of its own context only."""
+    keys, a function of its own context only.  An entry of several rows (a prompt's portion) goes, `tiles` allowing, to
+    workgroups of four waves that take four column tiles each and read the keys once for all of them; the same bits."""
     blocks = tuple(-(-c // LATENT_SPLIT_KEYS) if n == 1 else 1 for n, c in zip(row_counts, contexts)) if contexts is not None else None
-    key = (tuple(row_counts), heads, blocks, str(device))
+    key = (tuple(row_counts), heads, blocks, bool(tiles), str(device))
     plan = _LATENT_PLANS.get(key)
     if plan is None:
-        items, merges, row0, slot = [], [], 0, 0
+        wide, single, items, merges, row0, slot = [], [], [], [], 0, 0
         per = max(1, 16 // heads)
         for i, n in enumerate(row_counts):
             nb = blocks[i] if blocks is not None else 1
+            if n <= 0:
+                continue
+            if tiles and n > per:      # more rows than one column tile holds
+                span = per * LATENT_TILES
+                for r in range(((n - 1) // span) * span, -1, -span):
+                    for h0 in range(0, heads, 16):
+                        wide.append([row0 + r, min(span, n - r), h0, min(16, heads - h0), 0, 0, -1, 0])
+                row0 += n
+                continue
             for r in range(((n - 1) // per) * per, -1, -per):
                 for h0 in range(0, heads, 16):
                     nh = min(16, heads - h0)
+                    to = single if (tiles and n == 1) else items      # a decoded row's items go to workgroups of four waves
                     if nb <= 1:
-                        items.append([row0 + r, min(per, n - r), h0, nh, 0, 0, -1, 0])
+                        to.append([row0 + r, min(per, n - r), h0, nh, 0, 0, -1, 0])
                         continue
                     merges.append([row0, h0, nh, slot, nb, 0, 0, 0])
                     for b in range(nb):
-                        items.append([row0, 1, h0, nh, b * LATENT_SPLIT_KEYS, (b + 1) * LATENT_SPLIT_KEYS, slot + b, 0])
+                        to.append([row0, 1, h0, nh, b * LATENT_SPLIT_KEYS, (b + 1) * LATENT_SPLIT_KEYS, slot + b, 0])
                     slot += nb
             row0 += n
         if len(_LATENT_PLANS) > 256:
             _LATENT_PLANS.clear()
-        plan = _LATENT_PLANS[key] = LatentPlan(items, merges, slot, heads, row0, device)
+        plan = _LATENT_PLANS[key] = LatentPlan(wide, single, items, merges, slot, heads, row0, device)
     return plan
 
 

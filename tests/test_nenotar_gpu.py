@@ -170,7 +170,7 @@ def test_gated_recurrence_in_chunks():
     assert ops().scan_plan([255, 1, 30], "cuda") is None
 
 
-def _latent_case(seed, H, D, R, V, C, dims, scaling, positions, page, dtype, sharp=None):
+def _latent_case(seed, H, D, R, V, C, dims, scaling, positions, page, dtype, sharp=None, tiles=True):
     """One latent-attention layer on the kernels (products by torch) for rows at `positions` of one request whose earlier
     tokens are already cached in shuffled pages, against plain.latent_attention over the whole sequence."""
     from llmx_amd.parts.position import scaled_table
@@ -225,9 +225,10 @@ def _latent_case(seed, H, D, R, V, C, dims, scaling, positions, page, dtype, sha
         mixed = torch.empty(H, T, C, dtype=dtype, device="cuda")
         o.take_launches()
         o.latent_attention(q_lat, q_rot, cache, pos, entry, tables, mixed, 0.3, cache_t=cache_t,
-                           plan=o.latent_plan([0, T], H, "cuda", contexts=[0, max(rows) + 1]) if cores else None)
+                           plan=o.latent_plan([0, T], H, "cuda", contexts=[0, max(rows) + 1], tiles=tiles) if cores else None)
         ran = o.take_launches()
-        assert ("latent_attention.mfma" in ran) == cores
+        assert any(k in ran for k in ("latent_attention.mfma", "latent_attention.tiles", "latent_attention.rows")) == cores
+        assert not cores or tiles or set(ran) <= {"latent_attention.mfma", "latent_attention.merge"}
         assert ("latent_attention.merge" in ran) == (cores and T == 1 and max(rows) >= o.LATENT_SPLIT_KEYS)
         values = torch.bmm(mixed.float(), uv.float().transpose(1, 2)).contiguous()
         joined = torch.empty(T, H * V, dtype=dtype, device="cuda")
@@ -246,6 +247,9 @@ def test_latent_attention_rows_at_page_borders_and_first_tokens(dtype, sizes):
     positions = [0, 1, 2, 15, 16, 17, 63, 64, 65, 127, 128, 129, 200]
     got, want = _latent_case(11, H, D, R, V, C, dims, scaling, positions, 16, dtype)
     close(got, want, 3e-5 if dtype == torch.float32 else 3e-2)
+    if ops().latent_attention_mfma_ok(dtype, C, R, 16):
+        # the workgroups of four waves give every column the bits of the one-wave form
+        assert torch.equal(_latent_case(11, H, D, R, V, C, dims, scaling, positions, 16, dtype, tiles=False)[0], got)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["float32", "bfloat16"])
@@ -259,6 +263,8 @@ def test_latent_attention_finds_one_far_key(dtype, far):
     # the same row decoded alone: in bfloat16 its context is shared out over work items and joined
     got, want = _latent_case(5 + far, 2, 16, 32, 12, 32, 4, None, [n - 1], 16, dtype, sharp=(n - 1, far))
     close(got, want, 1e-4 if dtype == torch.float32 else 3e-2)
+    if dtype == torch.bfloat16:
+        assert torch.equal(_latent_case(5 + far, 2, 16, 32, 12, 32, 4, None, [n - 1], 16, dtype, sharp=(n - 1, far), tiles=False)[0], got)
 
 
 # ---------------------------------------------------------------------------
