@@ -22,8 +22,8 @@ def assemble(c: NenotarConfig) -> ModelSpec:
     n_layers = len(c.layers)
     side_width = (c.token_side_dim or 0) * n_layers
 
-    def norm(name):
-        return PartSpec("rmsnorm", {"width": E, "eps": c.norm_eps, "gain": "scalar", "tensor": ""}, name)
+    def norm(name, optional=False):
+        return PartSpec("rmsnorm", {"width": E, "eps": c.norm_eps, "gain": "scalar", "tensor": "", "optional": optional}, name)
 
     blocks = []
     for i, layer in enumerate(c.layers):
@@ -45,6 +45,9 @@ def assemble(c: NenotarConfig) -> ModelSpec:
             ffn = PartSpec("dense_act", {"hidden": E, "intermediate": layer.ff, "activation": "xielu"}, p + "mlp.")
             ffn_norm = norm(p + "norm2")
             extra["ffn_scale"] = ("scale", PartSpec("layer_scale", {"width": E}, p + "ls2"))
+        else:   # a file may hold the second norm and scale of a layer without a feed-forward: taken, never applied
+            ffn_norm = norm(p + "norm2", optional=True)
+            extra["ffn_scale"] = ("scale", PartSpec("layer_scale", {"width": E, "optional": True}, p + "ls2"))
         if c.token_side_dim:
             extra["token_input"] = ("token_input", PartSpec("gated_table", {
                 "hidden": E, "dim": c.token_side_dim, "column0": i * c.token_side_dim, "table": SIDE_TABLE, "table_width": side_width,

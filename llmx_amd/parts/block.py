@@ -50,19 +50,23 @@ class PreNormBlock:
 
 
 class LayerScale(Part):
-    """One learned factor a coordinate on a part's result.  params: width; tensor: the prefix itself, (width,)."""
+    """One learned factor a coordinate on a part's result.  params: width; optional (True: nothing applies it, and it is
+    listed only when the file holds it).  Tensor: the prefix itself, (width,)."""
     graph_safe = True
 
     def __init__(self, params, prefix, ctx):
         super().__init__(params, prefix, ctx)
         self.width = int(params["width"])
+        self.optional = bool(params.get("optional", False))
         self.weight = None
 
     def tensor_specs(self, available):
+        if self.optional and self.prefix not in available:
+            return []
         return [TensorSpec(self.prefix, (self.width,), "norm")]
 
     def load(self, tensors):
-        self.weight = tensors[self.prefix]
+        self.weight = tensors.get(self.prefix) if self.optional else tensors[self.prefix]
 
 
 class ParallelBlock:
@@ -73,8 +77,8 @@ class ParallelBlock:
     graph_safe = True
 
     def __init__(self, spec: BlockSpec, ctx: BuildContext):
-        if (spec.ffn is None) != (spec.ffn_norm is None):
-            raise ValueError("parallel block: a feed-forward and its norm come together")
+        if spec.ffn is not None and spec.ffn_norm is None:
+            raise ValueError("parallel block: a feed-forward comes with its norm")
         self.mixer_norm = build_part("norm", spec.mixer_norm, ctx)
         self.mixer = build_part("mixer", spec.mixer, ctx)
         self.ffn_norm = build_part("norm", spec.ffn_norm, ctx) if spec.ffn_norm is not None else None
@@ -90,14 +94,18 @@ class ParallelBlock:
         if unknown:
             raise ValueError(f"parallel block: no slot named {sorted(unknown)}")
         self.mixer_scale = built.get("mixer_scale")
-        self.ffn_scale = built.get("ffn_scale") if self.ffn is not None else None
+        self.ffn_scale = built.get("ffn_scale")
+        # without a feed-forward its norm and scale run nowhere; they may still be listed (as optional parts) for files that hold them
+        self._idle = [p for p in (self.ffn_norm, self.ffn_scale) if p is not None] if self.ffn is None else []
+        if self.ffn is None:
+            self.ffn_norm = self.ffn_scale = None
         self.token_input = built.get("token_input")
         a, b = self.mixer_norm, self.ffn_norm
         self._one_pass = isinstance(a, RMSNorm) and (b is None or (isinstance(b, RMSNorm) and b.eps == a.eps and b.width == a.width))
 
     def parts(self):
         return [p for p in (self.mixer_norm, self.mixer, self.ffn_norm, self.ffn, self.mixer_scale, self.ffn_scale, self.token_input)
-                if p is not None]
+                if p is not None] + self._idle
 
     def forward(self, step, x: torch.Tensor, cache: LayerCache) -> None:
         T, E = x.shape

@@ -17,7 +17,8 @@ from .spec import TensorSpec
 
 class RMSNorm(Norm):
     """params: width, eps; gain ("vector", the default: one weight a coordinate; "scalar": the file holds one number for
-    all coordinates); tensor (the name's last part, "weight" by default; "" when the prefix is the whole name).
+    all coordinates); tensor (the name's last part, "weight" by default; "" when the prefix is the whole name); optional
+    (True: a norm that nothing runs, listed only so that a file which holds its tensor all the same is not refused).
     Tensor: <prefix><tensor>, (width,) or ()."""
     graph_safe = True
 
@@ -29,12 +30,17 @@ class RMSNorm(Norm):
         if self.gain not in ("vector", "scalar"):
             raise ValueError(f"norm gain {self.gain!r} is not one of ['scalar', 'vector']")
         self.tensor = str(params.get("tensor", "weight"))
+        self.optional = bool(params.get("optional", False))
         self.weight: Optional[torch.Tensor] = None
 
     def tensor_specs(self, available):
+        if self.optional and self.name(self.tensor) not in available:
+            return []
         return [TensorSpec(self.name(self.tensor), (self.width,) if self.gain == "vector" else (), "norm")]
 
     def load(self, tensors):
+        if self.optional and self.name(self.tensor) not in tensors:
+            return
         w = tensors[self.name(self.tensor)]
         # one number for all coordinates is kept as a row of that number, which every norm kernel takes as it is
         self.weight = w if self.gain == "vector" else w.reshape(1).expand(self.width).contiguous()

@@ -55,6 +55,13 @@ def test_assembly_names_every_tensor_once_with_its_shape():
     assert specs["l0.mlp.up"].shape == (112, E) and specs["l0.mlp.act"].shape == (2,) and specs["l4.side.proj"].shape == (E, side)
     # a layer without a feed-forward has neither its norm nor its scale
     assert "l2.norm2" not in specs and "l2.ls2" not in specs and "l2.mlp.up" not in specs and "l3.norm2" not in specs
+    # ... unless the file holds them all the same: then they are taken (and never applied) rather than refused
+    from llmx_amd.engine.model import BuiltModel
+    from llmx_amd.models import registry
+    from llmx_amd.parts.base import BuildContext
+    model = BuiltModel(registry.assemble(read_config(copy.deepcopy(CONFIG_P))), BuildContext(torch.float32, torch.device("cpu"), 1))
+    held = {s.name for s in model.tensor_specs({"l2.norm2", "l2.ls2"})}
+    assert {"l2.norm2", "l2.ls2"} <= held and "l3.norm2" not in held
     # the folder written from these specs is what the plain implementation reads
     cfg, w = plain.load_folder(model_folder("P"))
     assert set(w) == set(specs) and all(tuple(w[n].shape) == tuple(specs[n].shape) for n in specs)
