@@ -93,7 +93,7 @@ extern "C" int llmx_latent_prep(const float* proj, const float* norm_w, const fl
 // The universal kernel: one wave per (row, head).  Keys lo..p of the row's request are walked in tiles of 64 absolute
 // positions with an online softmax; lane j of a tile forms the score of key 64*tile + j, for the weighted sum lane d
 // owns latent dims d, d + 64, ... and walks the tile's keys in order.  A row's arithmetic depends on its own position
-// and request only.  Any sizes with C <= 1024 and C + R <= 1536, float32 or bfloat16.
+// and request only.  Any sizes with C <= 2048 and C + R <= 4096, float32 or bfloat16.
 struct LatentAttnArgs {
     const void* q_lat;   // [H, T, C]
     const void* q_rot;   // [H, T, R]
@@ -106,8 +106,8 @@ struct LatentAttnArgs {
     int T, H, C, R, page_tokens, max_blocks, window;
 };
 
-#define LAT_MAX_C 1024
-#define LAT_MAX_CR 1536
+#define LAT_MAX_C 2048
+#define LAT_MAX_CR 4096
 
 template <typename T>
 __global__ void __launch_bounds__(64) latent_attention_generic_kernel(LatentAttnArgs a) {

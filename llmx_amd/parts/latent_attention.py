@@ -19,8 +19,8 @@ from .. import ops
 from .base import BuildContext, LayerCache, Mixer, build_part, register
 from .spec import CacheTensor, PagedNeed, PartSpec, TensorSpec
 
-MAX_LATENT = 1024          # the attention kernels keep a row's weighted sum of latents in a wave's registers
-MAX_LATENT_KEY = 1536      # latent + rotated key part: a query row in a workgroup's LDS
+MAX_LATENT = 2048          # the attention kernels keep a row's weighted sum of latents in a wave's registers
+MAX_LATENT_KEY = 4096      # latent + rotated key part: a query row in a workgroup's LDS
 
 
 class LatentAttention(Mixer):

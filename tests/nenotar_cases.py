@@ -57,9 +57,14 @@ CONFIG_R = {
         _layer("latent_attention", _latent(4, 32, 32, 24, 64, 0.125, 50000.0, 32), 48),
     ],
 }
-CONFIGS = {"P": CONFIG_P, "Q": CONFIG_Q, "R": CONFIG_R}
-PAGES = {"P": 16, "Q": 4, "R": 16}
-SEEDS = {"P": 3, "Q": 4, "R": 5}
+# S: recurrent layers only (no pages at all), one of them without a feed-forward.
+CONFIG_S = {
+    "architecture": "Nenotar", "vocab": 64, "width": 48, "embedding": {"scale": 2.0}, "norm": {"eps": 1e-6}, "token_side": {"dim": 8},
+    "layers": [_layer("mingru", {"width": 56}, 40), _layer("mingru", {"width": 24}, None)],
+}
+CONFIGS = {"P": CONFIG_P, "Q": CONFIG_Q, "R": CONFIG_R, "S": CONFIG_S}
+PAGES = {"P": 16, "Q": 4, "R": 16, "S": 16}
+SEEDS = {"P": 3, "Q": 4, "R": 5, "S": 6}
 
 
 def write_folder(config: dict, seed: int, folder: str, edit=None) -> str:
