@@ -23,7 +23,9 @@ CONTEXT = 4096
 SIZES = {
     "w2048": (2048, 8, 16, 8192, 3072, 128, 32768),
     "w4096": (4096, 4, 32, 16384, 6144, 256, 32768),
+    "w256": (256, 2, 2, 768, 384, 16, 1024),        # seconds: for trying the option out; not among the default sizes
 }
+DEFAULT_SIZES = ("w2048", "w4096")
 
 
 def nenotar_config(width, layers, heads, ff, recurrent, side, vocab):
@@ -153,7 +155,9 @@ def run(design: str, steps: int, warmup: int, sizes=None) -> dict:
         raise SystemExit(f"bench: no design named {design!r} (known: nenotar)")
     result = {"design": "Nenotar", "closest": "MiniMax-M3 (GQA attention, routed SwiGLU experts)", "dtype": "bf16", "prompt": PROMPT,
               "context": CONTEXT, "data": "synthetic: LCG token ids, N(0,0.02) weights generated on the device", "sizes": {}}
-    for name in (sizes or SIZES):
+    for name in (sizes or DEFAULT_SIZES):
+        if name not in SIZES:
+            raise SystemExit(f"bench: no size named {name!r} (known: {sorted(SIZES)})")
         shape = SIZES[name]
         per = {}
         for which, make in (("nenotar", nenotar_config), ("closest", closest_config)):

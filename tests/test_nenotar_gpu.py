@@ -519,3 +519,23 @@ def test_trace_replay_and_command_line(tmp_path):
                          capture_output=True, text=True, timeout=600)
     assert cli.returncode == 0, cli.stderr[-2000:]
     assert int(cli.stdout.splitlines()[-1].split()[0]) == int(torch.argmax(want["b"][8]))
+
+
+def test_command_line_generates_from_a_configuration_with_random_weights(tmp_path):
+    """`llmx generate --config JSON --random SEED` for this design: weights generated on the device, the scheduler's loop,
+    the device sampler; the same seed gives the same tokens, greedy or drawn."""
+    import json
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    cfg = tmp_path / "config.json"
+    cfg.write_text(json.dumps(CONFIGS["P"]))
+    outs = []
+    for extra in (["--temp", "0"], ["--temp", "0"], ["--temp", "0.8", "--topk", "20", "--seed", "7"], ["--temp", "0.8", "--topk", "20", "--seed", "7"]):
+        run = subprocess.run([sys.executable, os.path.join(root, "bin", "llmx"), "generate", "--config", str(cfg), "--random", "5", "--std", "0.06",
+                              "3 1 4 1 5 9 2 6", "-n", "9"] + extra, capture_output=True, text=True, timeout=600)
+        assert run.returncode == 0, run.stderr[-2000:]
+        ids = [int(t) for t in run.stdout.split()]
+        assert len(ids) == 9 and all(0 <= t < CONFIGS["P"]["vocab"] for t in ids)
+        outs.append(ids)
+    assert outs[0] == outs[1] and outs[2] == outs[3]
