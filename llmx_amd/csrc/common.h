@@ -236,4 +236,36 @@ __device__ __forceinline__ void rms_rows_as_1024(const float* __restrict__ X, si
     }
 }
 
+// A one-argument activation that a product applies to what it stores (the store epilogue only), or a kernel of its own.
+// xIELU with two learned numbers (p, q) read from the device: z > 0: softplus(p) z^2 + z/2; z <= 0: (1/2 + softplus(q))
+// (e^z - 1 - z) + z/2.  Both go through these two functions, so a product with the activation gives the bits of the product
+// followed by the activation's kernel.
+enum : int { LLMX_ACT_NONE = 0, LLMX_ACT_XIELU = 1 };
+__device__ __forceinline__ float softplus_f(float v) { return log1pf(expf(-fabsf(v))) + fmaxf(v, 0.0f); }
+// The activation's numbers as a kernel reads them at its start (uniform loads, long before the epilogue needs them).
+struct ActParams {
+    float p, q;
+    __device__ __forceinline__ ActParams(int kind, const float* __restrict__ params) : p(0.0f), q(0.0f) {
+        if (kind != LLMX_ACT_NONE) {
+            p = params[0];
+            q = params[1];
+        }
+    }
+};
+struct ActFn {
+    int kind;
+    float a, b;
+    __device__ __forceinline__ ActFn(int kind_, const ActParams& at) : kind(kind_), a(0.0f), b(0.0f) {
+        if (kind == LLMX_ACT_XIELU) {
+            a = softplus_f(at.p);
+            b = 0.5f + softplus_f(at.q);
+        }
+    }
+    __device__ __forceinline__ ActFn(int kind_, const float* __restrict__ params) : ActFn(kind_, ActParams(kind_, params)) {}
+    __device__ __forceinline__ float operator()(float v) const {
+        if (kind == LLMX_ACT_XIELU) return v > 0.0f ? a * v * v + 0.5f * v : b * (expm1f(v) - v) + 0.5f * v;
+        return v;
+    }
+};
+
 #define LLMX_CHECK_LAUNCH() (int)hipGetLastError()

@@ -26,6 +26,8 @@ struct GemmArgs {
     int a_div;
     long w_group_stride;
     int up_offset;  // EPI_SWIGLU: W row n is the gate row, W row n + up_offset the up row
+    int act;        // EPI_STORE: an activation applied to what is stored (LLMX_ACT_*), with its parameters on the device
+    const float* act_params;
 };
 
 template <typename TA, typename TW, typename TC, int EPI>
@@ -50,6 +52,7 @@ __global__ void __launch_bounds__(256) gemm_generic_kernel(GemmArgs g) {
     const int tile_step = g.group_offsets ? GT_BM : GT_BM * gridDim.y;
     const int first = g.group_offsets ? row_begin : row_begin + blockIdx.y * GT_BM;
     const int tx = tid % 16, ty = tid / 16;
+    const ActFn act(EPI == EPI_STORE ? g.act : LLMX_ACT_NONE, g.act_params);
 
     for (int m0 = first; m0 < row_end; m0 += tile_step) {
         if (tid < GT_BM) {
@@ -130,6 +133,8 @@ __global__ void __launch_bounds__(256) gemm_generic_kernel(GemmArgs g) {
                     v = (v / (1.0f + expf(-v))) * accu[i][j];
                 } else if (EPI == EPI_ADD) {
                     v = ld(c) + v;
+                } else {
+                    v = act(v);
                 }
                 st(c, v);
             }
@@ -158,11 +163,13 @@ static int launch_c(const GemmArgs& g, int c_dtype, int epi, dim3 grid, hipStrea
 // dtype codes: 0 f32, 1 bf16.  n_groups == 0: dense product over M rows.  n_groups > 0: grouped (see GemmArgs).
 extern "C" int llmx_gemm_generic(const void* A, int a_dtype, const void* W, int w_dtype, void* C, int c_dtype, int M, int N, int K, int lda,
                                  int ldw, int ldc, int epi, int n_groups, const int* group_offsets, const int* list, int a_div,
-                                 long w_group_stride, int up_offset, hipStream_t stream) {
+                                 long w_group_stride, int up_offset, int act, const float* act_params, hipStream_t stream) {
     if (N <= 0 || K <= 0) return 0;
     if (n_groups == 0 && M <= 0) return 0;
     llmx_note_launch(n_groups ? LK_GEMM_GENERIC_GROUPED : LK_GEMM_GENERIC);
-    GemmArgs g{A, W, C, M, N, K, lda, ldw, ldc, n_groups ? group_offsets : nullptr, list, a_div > 0 ? a_div : 1, w_group_stride, up_offset};
+    GemmArgs g{A, W, C, M, N, K, lda, ldw, ldc, n_groups ? group_offsets : nullptr, list, a_div > 0 ? a_div : 1, w_group_stride, up_offset,
+               epi == EPI_STORE ? act : LLMX_ACT_NONE, act_params};
+    if (act != LLMX_ACT_NONE && (epi != EPI_STORE || !act_params)) return -2;
     dim3 grid;
     grid.x = (N + GT_BN - 1) / GT_BN;
     if (n_groups) {

@@ -41,6 +41,9 @@ struct SkinnyArgs {
     const float* norm_w;
     float norm_eps;
     int x_rows;
+    // SK_STORE: an activation applied to what is stored (LLMX_ACT_*), with its parameters on the device
+    int act;
+    const float* act_params;
 };
 
 __device__ __forceinline__ bf16x8_t load_frag(const bf16_t* p, bool in) {
@@ -61,6 +64,7 @@ __global__ void __launch_bounds__(64 * KS) gemm_skinny_kernel(SkinnyArgs g) {
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     const int r = lane & 15, kg = lane >> 4;
     const int n0 = blockIdx.x * 16;
+    const ActParams act_params(EPI == SK_STORE ? g.act : LLMX_ACT_NONE, g.act_params);
     const bf16_t* W = g.W;
     int row_begin = 0, row_end = g.M;
     if (GROUPED) {
@@ -226,6 +230,7 @@ __global__ void __launch_bounds__(64 * KS) gemm_skinny_kernel(SkinnyArgs g) {
                     float x = v[0][i];
                     if (EPI == SK_SWIGLU) x = (x / (1.0f + expf(-x))) * v[1][i];
                     if (EPI == SK_ADD) x = c_old[t][i] + x;
+                    if (EPI == SK_STORE && g.act != LLMX_ACT_NONE) x = ActFn(g.act, act_params)(x);
                     st(c + i, x);
                 }
             }
@@ -245,6 +250,7 @@ __global__ void __launch_bounds__(64 * KS) gemm_skinny_two_strips_kernel(SkinnyA
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     const int r = lane & 15, kg = lane >> 4;
     const int n0 = blockIdx.x * 32;
+    const ActParams act_params(EPI == SK_STORE ? g.act : LLMX_ACT_NONE, g.act_params);
     const int K = g.K;
     const int steps_total = (K + 31) >> 5;
     const int per = (steps_total + KS - 1) / KS;
@@ -313,6 +319,7 @@ __global__ void __launch_bounds__(64 * KS) gemm_skinny_two_strips_kernel(SkinnyA
                 if (n0 + 16 * q + 4 * kg + i >= g.N) continue;
                 float x = v[i];
                 if (EPI == SK_ADD) x = ld(c + i) + x;
+                if (EPI == SK_STORE && g.act != LLMX_ACT_NONE) x = ActFn(g.act, act_params)(x);
                 st(c + i, x);
             }
         }
@@ -403,7 +410,7 @@ extern "C" int llmx_gemm_skinny_normed_ok(int x_rows, int K) {
 extern "C" int llmx_gemm_skinny(const void* A, const void* W, void* C, int c_dtype, int M, int N, int K, int lda, int ldc, int epi, int ks,
                                 int n_groups, int max_active, const int* active, const int* n_active, const int* group_offsets,
                                 const int* list, int a_div, long w_group_stride, int up_offset, const float* X, const float* norm_w,
-                                float norm_eps, int x_rows, hipStream_t stream) {
+                                float norm_eps, int x_rows, int act, const float* act_params, hipStream_t stream) {
     if (N <= 0 || K <= 0) return 0;
     if (K % 8) return -2;
     const bool grouped = n_groups > 0;
@@ -411,7 +418,8 @@ extern "C" int llmx_gemm_skinny(const void* A, const void* W, void* C, int c_dty
     if (grouped && max_active <= 0) return 0;
     if (X && (!norm_w || epi == SK_ADD || !llmx_gemm_skinny_normed_ok(x_rows, K) || (!grouped && x_rows != M))) return -2;
     SkinnyArgs g{(const bf16_t*)A, (const bf16_t*)W, C, M, N, K, lda, ldc, active, n_active, group_offsets, list, a_div > 0 ? a_div : 1,
-                 w_group_stride, up_offset, X, norm_w, norm_eps, x_rows};
+                 w_group_stride, up_offset, X, norm_w, norm_eps, x_rows, epi == SK_STORE ? act : LLMX_ACT_NONE, act_params};
+    if (act != LLMX_ACT_NONE && (epi != SK_STORE || !act_params)) return -2;
     dim3 grid((N + 15) / 16, grouped ? max_active : 1, 1);
     int mt = 1;
     if (!grouped && epi != SK_SWIGLU) mt = M <= 16 ? 1 : (M <= 32 ? 2 : 4);

@@ -85,6 +85,8 @@ struct TileArgs {
     const int* tile_stats;  // grouped, optional: [0] = sum over groups of ceil(rows / 128)
     int run_if_big;         // with tile_stats: 1: this launch works only if the groups fill 128-row tiles, 0: only if not
     int run_tiles;          // dense lean form, > 0: workgroup z multiplies only K's run z (this many 64-wide tiles) and stores its sums at C + z * M * ldc
+    int act;                // TL_STORE: an activation applied to what is stored (LLMX_ACT_*; a launch of runs' sums leaves it to the kernel that adds them)
+    const float* act_params;
 };
 
 // Whether the groups' rows fill tiles of 128 rows well enough: the tiles hold at most 1.6 times the rows (measured on
@@ -447,7 +449,12 @@ __global__ void __launch_bounds__(256) gemm_tile_kernel(TileArgs g) {
         } else {
 #pragma unroll
             for (int f = 0; f < 4; ++f) {
-                const float v[4] = {acc[f][t][0], acc[f][t][1], acc[f][t][2], acc[f][t][3]};
+                float v[4] = {acc[f][t][0], acc[f][t][1], acc[f][t][2], acc[f][t][3]};
+                if (EPI == TL_STORE && g.act != LLMX_ACT_NONE) {
+                    const ActFn act(g.act, g.act_params);
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) v[i] = act(v[i]);
+                }
                 store_quad<EPI == TL_ADD>(crow, n0 + 64 * wn + 16 * f + fq, g.N, rows_aligned, v);
             }
         }
@@ -714,7 +721,12 @@ __global__ void __launch_bounds__(512) gemm_wide_kernel(TileArgs g) {
         } else {
 #pragma unroll
             for (int f = 0; f < 4; ++f) {
-                const float v[4] = {acc[f][q][0], acc[f][q][1], acc[f][q][2], acc[f][q][3]};
+                float v[4] = {acc[f][q][0], acc[f][q][1], acc[f][q][2], acc[f][q][3]};
+                if (EPI == TL_STORE && g.act != LLMX_ACT_NONE) {
+                    const ActFn act(g.act, g.act_params);
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) v[i] = act(v[i]);
+                }
                 store_quad<EPI == TL_ADD>(crow, n0 + 64 * wn + 16 * f + fq, g.N, rows_aligned, v);
             }
         }
@@ -773,7 +785,8 @@ extern "C" int llmx_gemm_tile_offsets_fit(int M, int N, int K, int lda, int epi,
 // The runs' sums of a product whose runs were multiplied apart (TileArgs::run_tiles), added in run order as the kernel
 // that holds all runs adds them, then stored as the epilogue says.  Four neighbouring features a thread.
 template <bool ADD, typename TC>
-__global__ void __launch_bounds__(256) gemm_runs_sum_kernel(const float* __restrict__ partial, TC* __restrict__ C, int M, int N, int ldc, int runs) {
+__global__ void __launch_bounds__(256) gemm_runs_sum_kernel(const float* __restrict__ partial, TC* __restrict__ C, int M, int N, int ldc, int runs,
+                                                          int act_kind, const float* __restrict__ act_params) {
     const int quads = (N + 3) / 4;
     const long at = (long)blockIdx.x * 256 + threadIdx.x;
     if (at >= (long)M * quads) return;
@@ -793,6 +806,11 @@ __global__ void __launch_bounds__(256) gemm_runs_sum_kernel(const float* __restr
         }
 #pragma unroll
         for (int i = 0; i < 4; ++i) v[i] = r == 0 ? x[i] : v[i] + x[i];
+    }
+    if (!ADD && act_kind != LLMX_ACT_NONE) {
+        const ActFn act(act_kind, act_params);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[i] = act(v[i]);
     }
     store_quad<ADD>(C + (size_t)m * ldc, n, N, ldc % 4 == 0 && ((uintptr_t)C & 15) == 0, v);
 }
@@ -826,7 +844,7 @@ extern "C" long llmx_gemm_tile_runs_scratch(int M, int N, int K, int epi, int ks
 
 extern "C" int llmx_gemm_tile(const void* A, const void* W, void* C, int c_dtype, int M, int N, int K, int lda, int ldc, int epi, int ks,
                               int n_groups, int max_tiles, const int* group_offsets, const int* list, int a_div, long w_group_stride,
-                              int up_offset, const int* tile_stats, float* runs_scratch, hipStream_t stream) {
+                              int up_offset, const int* tile_stats, float* runs_scratch, int act, const float* act_params, hipStream_t stream) {
     if (M <= 0 || N <= 0 || K <= 0) return 0;
     if (K % 8) return -2;
     const bool grouped = n_groups > 0;
@@ -834,7 +852,8 @@ extern "C" int llmx_gemm_tile(const void* A, const void* W, void* C, int c_dtype
     const int steps = (K + 31) / 32, per = (steps + ks - 1) / ks;
     const bool lean = K % TL_BK == 0 && (ks == 1 || per % 2 == 0) && llmx_gemm_tile_offsets_fit(M, N, K, lda, epi, n_groups, a_div, up_offset);
     TileArgs g{(const bf16_t*)A, (const bf16_t*)W, C, M, N, K, lda, ldc, group_offsets, list, n_groups, a_div > 0 ? a_div : 1,
-               w_group_stride, up_offset, 0, ks, 64, nullptr, 0, 0};
+               w_group_stride, up_offset, 0, ks, 64, nullptr, 0, 0, epi == TL_STORE ? act : LLMX_ACT_NONE, act_params};
+    if (act != LLMX_ACT_NONE && (epi != TL_STORE || !act_params)) return -2;
     auto launch = [&](int form, int tiles_y) -> int {
         g.bm = form_rows(form);
         g.m_tiles = (M + g.bm - 1) / g.bm;
@@ -860,6 +879,7 @@ extern "C" int llmx_gemm_tile(const void* A, const void* W, void* C, int c_dtype
         part.bm = 64;
         part.m_tiles = (M + 63) / 64;
         part.run_tiles = tiles_per_run;
+        part.act = LLMX_ACT_NONE;       // the runs' sums are stored bare; the kernel that adds them applies the activation
         llmx_note_launch(LK_GEMM_TILE_RUNS_APART);
         hipLaunchKernelGGL((gemm_tile_kernel<TL_STORE, float, false, false, true, 64>), dim3((N + TL_BN - 1) / TL_BN, part.m_tiles, runs), dim3(256), 0,
                            stream, part);
@@ -867,11 +887,11 @@ extern "C" int llmx_gemm_tile(const void* A, const void* W, void* C, int c_dtype
         const dim3 sum_grid((unsigned)((quads + 255) / 256));
         if (epi == TL_ADD) {
             if (c_dtype != LLMX_F32) return -2;
-            hipLaunchKernelGGL((gemm_runs_sum_kernel<true, float>), sum_grid, dim3(256), 0, stream, (const float*)runs_scratch, (float*)C, M, N, ldc, runs);
+            hipLaunchKernelGGL((gemm_runs_sum_kernel<true, float>), sum_grid, dim3(256), 0, stream, (const float*)runs_scratch, (float*)C, M, N, ldc, runs, 0, nullptr);
         } else if (c_dtype == LLMX_BF16) {
-            hipLaunchKernelGGL((gemm_runs_sum_kernel<false, bf16_t>), sum_grid, dim3(256), 0, stream, (const float*)runs_scratch, (bf16_t*)C, M, N, ldc, runs);
+            hipLaunchKernelGGL((gemm_runs_sum_kernel<false, bf16_t>), sum_grid, dim3(256), 0, stream, (const float*)runs_scratch, (bf16_t*)C, M, N, ldc, runs, g.act, g.act_params);
         } else {
-            hipLaunchKernelGGL((gemm_runs_sum_kernel<false, float>), sum_grid, dim3(256), 0, stream, (const float*)runs_scratch, (float*)C, M, N, ldc, runs);
+            hipLaunchKernelGGL((gemm_runs_sum_kernel<false, float>), sum_grid, dim3(256), 0, stream, (const float*)runs_scratch, (float*)C, M, N, ldc, runs, g.act, g.act_params);
         }
         rc = 0;
     } else if (!grouped) {

@@ -88,27 +88,21 @@ extern "C" int llmx_rmsnorm_add(float* x, const float* y, const float* w, float 
 
 // ---------------------------------------------------------------------------
 // Activations between two products, float32 in, the activation type out.
-__device__ __forceinline__ float softplus_f(float v) { return log1pf(expf(-fabsf(v))) + fmaxf(v, 0.0f); }
-
 // xIELU with the two numbers (p, q) of `pq`: z > 0: softplus(p) z^2 + z/2; z <= 0: (1/2 + softplus(q)) (e^z - 1 - z) + z/2.
-__device__ __forceinline__ float xielu_f(float v, float up, float down) {
-    return v > 0.0f ? up * v * v + 0.5f * v : down * (expm1f(v) - v) + 0.5f * v;
-}
-
 // Four neighbouring values a thread (one 16-byte load); the last thread takes what is left one by one.
 template <typename TO>
 __global__ void __launch_bounds__(256) xielu_kernel(const float* __restrict__ z, const float* __restrict__ pq, TO* __restrict__ out, size_t total) {
     typedef float f32x4_t __attribute__((ext_vector_type(4)));
     const size_t at = 4 * ((size_t)blockIdx.x * 256 + threadIdx.x);
     if (at >= total) return;
-    const float up = softplus_f(pq[0]), down = 0.5f + softplus_f(pq[1]);
+    const ActFn act(LLMX_ACT_XIELU, pq);
     if (at + 4 <= total) {
         const f32x4_t v = *reinterpret_cast<const f32x4_t*>(z + at);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) st(out + at + i, xielu_f(v[i], up, down));
+        for (int i = 0; i < 4; ++i) st(out + at + i, act(v[i]));
         return;
     }
-    for (size_t i = at; i < total; ++i) st(out + i, xielu_f(z[i], up, down));
+    for (size_t i = at; i < total; ++i) st(out + i, act(z[i]));
 }
 
 extern "C" int llmx_act_xielu(const float* z, const float* pq, void* out, int out_dtype, long total, hipStream_t stream) {

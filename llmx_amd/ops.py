@@ -72,19 +72,19 @@ def _declare(h) -> None:
         "llmx_fill_random": [P, I, L, ctypes.c_ulonglong, I, F, F, P],
         "llmx_read_probe": [P, L, P, P],
         "llmx_attention_partial_pad": [],
-        "llmx_gemm_generic": [P, I, P, I, P, I, I, I, I, I, I, I, I, I, P, P, I, L, I, P],
+        "llmx_gemm_generic": [P, I, P, I, P, I, I, I, I, I, I, I, I, I, P, P, I, L, I, I, P, P],
         "llmx_qknorm_rope_kvwrite": [P, P, P, P, P, P, P, P, P, P, I, F, I, I, I, I, I, I, I, I, I, I, P],
         "llmx_paged_attention_generic": [P, P, P, P, P, P, P, I, F, I, I, I, I, I, I, I, P],
         "llmx_paged_attention_mfma": [P, P, P, P, P, P, P, I, I, I, P, I, P, P, P, F, I, I, I, I, I, I, I, P],
         "llmx_route_topk": [P, P, I, L, P, P, P, I, I, I, I, I, F, P],
         "llmx_moe_align": [P, I, I, P, P, P, P, P, P, P, P],
         "llmx_route_topk_align": [P, P, I, L, P, P, P, I, I, I, I, F, P, P, P, P, P, P],
-        "llmx_gemm_skinny": [P, P, P, I, I, I, I, I, I, I, I, I, I, P, P, P, P, I, L, I, P, P, F, I, P],
+        "llmx_gemm_skinny": [P, P, P, I, I, I, I, I, I, I, I, I, I, P, P, P, P, I, L, I, P, P, F, I, I, P, P],
         "llmx_gemm_skinny_normed_ok": [I, I],
         "llmx_gemm_skinny_f32_normed_ok": [I, I],
         "llmx_argmax_rows": [P, P, P, P, I, I, P],
         "llmx_gemm_skinny_f32": [P, P, P, I, I, I, I, I, I, I, I, L, P, F, P],
-        "llmx_gemm_tile": [P, P, P, I, I, I, I, I, I, I, I, I, I, P, P, I, L, I, P, P, P],
+        "llmx_gemm_tile": [P, P, P, I, I, I, I, I, I, I, I, I, I, P, P, I, L, I, P, P, I, P, P],
         "llmx_gemm_tile_offsets_fit": [I, I, I, I, I, I, I, I],
         "llmx_sample_all": [P, P, P, P, P, P, I, I, P, P],
         "llmx_sample_topk": [P, P, P, P, P, P, P, P, I, I, P, I, P],
@@ -527,12 +527,22 @@ def gemm_f32_takes_normed_rows(rows: int, w: torch.Tensor) -> bool:
     return rows <= NORMED_ROWS_PAY and gemm_f32_can_norm_rows(rows, w)
 
 
-def gemm(a, w: torch.Tensor, c: torch.Tensor, epilogue: int = EPI_STORE, force_generic: bool = False, scratch=None) -> None:
+ACT_NONE, ACT_XIELU = 0, 1      # activations a storing product can apply to what it stores
+
+
+def gemm(a, w: torch.Tensor, c: torch.Tensor, epilogue: int = EPI_STORE, force_generic: bool = False, scratch=None, act=None) -> None:
     """c[M,N] (+)= a[M,K] @ w[N,K]^T, accumulated in float32; EPI_SWIGLU: c = silu(a @ w[:N]^T) * (a @ w[N:]^T).
     `a` may be NormedRows where gemm_takes_normed_rows says so: the product reads bfloat16(norm(x)).
     `scratch(name, shape, dtype)` gives storage that lives as long as the caller's step (a step's workspace): with it,
-    products of some tens of rows multiply K's runs in workgroups of their own; the bits are the same either way."""
+    products of some tens of rows multiply K's runs in workgroups of their own; the bits are the same either way.
+    `act` = (ACT_XIELU, params): with EPI_STORE, c = activation(a @ w^T), params the activation's numbers on the device
+    (xIELU: float32 (p, q)); the bits of the product followed by the activation's own kernel (act_xielu)."""
     M, K = a.shape
+    act_args = (0, 0)
+    if act is not None:
+        if epilogue != EPI_STORE or act[0] != ACT_XIELU:
+            raise KernelError("gemm: an activation goes with the store epilogue, and xIELU is the one built")
+        act_args = (ACT_XIELU, _dev(act[1], "activation parameters", torch.float32, (2,)))
     N = w.shape[0] // 2 if epilogue == EPI_SWIGLU else w.shape[0]   # swiglu: w holds gate rows, then up rows
     if w.shape[1] != K or tuple(c.shape) != (M, N):
         raise KernelError(f"gemm shapes do not agree: a {tuple(a.shape)}, w {tuple(w.shape)}, c {tuple(c.shape)}")
@@ -540,7 +550,7 @@ def gemm(a, w: torch.Tensor, c: torch.Tensor, epilogue: int = EPI_STORE, force_g
         if not gemm_can_norm_rows(M, w, c.dtype, epilogue):
             raise KernelError("gemm: normed rows are not taken for this product")
         _check(lib().llmx_gemm_skinny(0, _dev(w, "w"), _dev(c, "c"), _code(c.dtype), M, N, K, K, N, epilogue,
-                                      _split_k(-(-N // 16), K), 0, 0, 0, 0, 0, 0, 1, 0, N if epilogue == EPI_SWIGLU else 0, *a.args(), _stream()),
+                                      _split_k(-(-N // 16), K), 0, 0, 0, 0, 0, 0, 1, 0, N if epilogue == EPI_SWIGLU else 0, *a.args(), *act_args, _stream()),
                "gemm_skinny (normed rows)")
         return
     # a product wide enough to fill the chip with tiles (the LM head) streams its weights faster through the tiled kernel
@@ -557,16 +567,16 @@ def gemm(a, w: torch.Tensor, c: torch.Tensor, epilogue: int = EPI_STORE, force_g
         skinny = False
     if not force_generic and skinny and _skinny_ok(a, w, c, epilogue):
         _check(lib().llmx_gemm_skinny(_dev(a, "a"), _dev(w, "w"), _dev(c, "c"), _code(c.dtype), M, N, K, K, N, epilogue,
-                                      _split_k(-(-N // 16), K), 0, 0, 0, 0, 0, 0, 1, 0, N if epilogue == EPI_SWIGLU else 0, *_NO_NORM, _stream()),
+                                      _split_k(-(-N // 16), K), 0, 0, 0, 0, 0, 0, 1, 0, N if epilogue == EPI_SWIGLU else 0, *_NO_NORM, *act_args, _stream()),
                "gemm_skinny")
         return
     if not force_generic and _skinny_ok(a, w, c, epilogue):
         runs = scratch("gemm_tile.runs", (runs_apart,), torch.float32) if runs_apart else None
         _check(lib().llmx_gemm_tile(_dev(a, "a"), _dev(w, "w"), _dev(c, "c"), _code(c.dtype), M, N, K, K, N, epilogue,
-                                    ks, 0, 0, 0, 0, 1, 0, N if epilogue == EPI_SWIGLU else 0, 0, _dev(runs, "runs"), _stream()), "gemm_tile")
+                                    ks, 0, 0, 0, 0, 1, 0, N if epilogue == EPI_SWIGLU else 0, 0, _dev(runs, "runs"), *act_args, _stream()), "gemm_tile")
         return
     _check(lib().llmx_gemm_generic(_dev(a, "a"), _code(a.dtype), _dev(w, "w"), _code(w.dtype), _dev(c, "c"), _code(c.dtype),
-                                   M, N, K, K, K, N, epilogue, 0, 0, 0, 1, 0, N if epilogue == EPI_SWIGLU else 0, _stream()), "gemm")
+                                   M, N, K, K, K, N, epilogue, 0, 0, 0, 1, 0, N if epilogue == EPI_SWIGLU else 0, *act_args, _stream()), "gemm")
 
 
 def grouped_gemm(a: torch.Tensor, w: torch.Tensor, c: torch.Tensor, offsets: torch.Tensor, pairs: torch.Tensor, a_div: int,
@@ -593,7 +603,7 @@ def grouped_gemm(a: torch.Tensor, w: torch.Tensor, c: torch.Tensor, offsets: tor
         _check(lib().llmx_gemm_skinny(0, _dev(w, "w"), _dev(c, "c"), _code(c.dtype), n_pairs, N, K, K, N, epilogue,
                                       _split_k(-(-N // 16), K), G, min(G, n_pairs), _dev(active, "active", torch.int32, (G,)),
                                       _dev(n_active, "n_active", torch.int32, (1,)), _dev(offsets, "offsets", torch.int32, (G + 1,)),
-                                      _dev(pairs, "pairs", torch.int32), a_div, NW * K, N if epilogue == EPI_SWIGLU else 0, *a.args(), _stream()),
+                                      _dev(pairs, "pairs", torch.int32), a_div, NW * K, N if epilogue == EPI_SWIGLU else 0, *a.args(), 0, 0, _stream()),
                "grouped_gemm_skinny (normed rows)")
         return
     if (not force_generic and active is not None and n_active is not None and _skinny_ok(a, w, c, epilogue)
@@ -601,19 +611,19 @@ def grouped_gemm(a: torch.Tensor, w: torch.Tensor, c: torch.Tensor, offsets: tor
         _check(lib().llmx_gemm_skinny(_dev(a, "a"), _dev(w, "w"), _dev(c, "c"), _code(c.dtype), n_pairs, N, K, K, N, epilogue,
                                       _split_k(-(-N // 16), K), G, min(G, n_pairs), _dev(active, "active", torch.int32, (G,)),
                                       _dev(n_active, "n_active", torch.int32, (1,)), _dev(offsets, "offsets", torch.int32, (G + 1,)),
-                                      _dev(pairs, "pairs", torch.int32), a_div, NW * K, N if epilogue == EPI_SWIGLU else 0, *_NO_NORM, _stream()),
+                                      _dev(pairs, "pairs", torch.int32), a_div, NW * K, N if epilogue == EPI_SWIGLU else 0, *_NO_NORM, 0, 0, _stream()),
                "grouped_gemm_skinny")
         return
     if not force_generic and _skinny_ok(a, w, c, epilogue):
         _check(lib().llmx_gemm_tile(_dev(a, "a"), _dev(w, "w"), _dev(c, "c"), _code(c.dtype), n_pairs, N, K, K, N, epilogue,
                                     _split_k(-(-N // 16), K), G, min(G, n_pairs) + n_pairs // 64, _dev(offsets, "offsets", torch.int32, (G + 1,)),
                                     _dev(pairs, "pairs", torch.int32), a_div, NW * K, N if epilogue == EPI_SWIGLU else 0,
-                                    _dev(tile_stats if n_pairs >= TILE_STATS_MIN_PAIRS else None, "tile_stats", torch.int32, (1,)), 0, _stream()),
+                                    _dev(tile_stats if n_pairs >= TILE_STATS_MIN_PAIRS else None, "tile_stats", torch.int32, (1,)), 0, 0, 0, _stream()),
                "grouped_gemm_tile")
         return
     _check(lib().llmx_gemm_generic(_dev(a, "a"), _code(a.dtype), _dev(w, "w"), _code(w.dtype), _dev(c, "c"), _code(c.dtype),
                                    n_pairs, N, K, K, K, N, epilogue, G, _dev(offsets, "offsets", torch.int32, (G + 1,)),
-                                   _dev(pairs, "pairs", torch.int32), a_div, NW * K, N if epilogue == EPI_SWIGLU else 0, _stream()),
+                                   _dev(pairs, "pairs", torch.int32), a_div, NW * K, N if epilogue == EPI_SWIGLU else 0, 0, 0, _stream()),
            "grouped_gemm")
 
 

@@ -165,10 +165,8 @@ class DenseAct(FeedForward):
         self.act = tensors[self.name("act")]
 
     def forward(self, step, h, out, accumulate, h32=None):
-        z = step.buf("dense.pre", (step.rows, self.intermediate), torch.float32)
-        ops.gemm(h, self.w_up, z, scratch=step.buf)
         a = step.buf("dense.act", (step.rows, self.intermediate), step.act_dtype)
-        ops.act_xielu(z, self.act, a)
+        ops.gemm(h, self.w_up, a, scratch=step.buf, act=(ops.ACT_XIELU, self.act))      # the activation in the product's epilogue
         ops.gemm(a, self.w_down, out, ops.EPI_ADD if accumulate else ops.EPI_STORE, scratch=step.buf)
 
 

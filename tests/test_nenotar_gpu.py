@@ -102,6 +102,35 @@ def test_xielu_both_branches_and_the_gated_table_slice():
         close(out, want, 1e-6)
 
 
+@pytest.mark.parametrize("M,N,K,dtype", [(1, 48, 64, "bf16"), (3, 200, 256, "bf16"), (40, 4096, 256, "bf16"), (40, 130, 512, "bf16"), (300, 96, 128, "bf16"),
+                                         (2048, 3072, 256, "bf16"), (5, 33, 54, "bf16"), (70, 50, 48, "f32")])
+def test_activation_in_the_products_epilogue(M, N, K, dtype):
+    """A storing product with xIELU gives the bits of the product followed by the activation's kernel, in every form of the
+    product (weight streaming, two strips, tiles, wide tiles, K's runs apart, the universal kernel), and the plain values."""
+    o = ops()
+    g = torch.Generator().manual_seed(M + N + K)
+    t = torch.bfloat16 if dtype == "bf16" else torch.float32
+    a, w = dev(torch.randn(M, K, generator=g), t), dev(torch.randn(N, K, generator=g) * 0.3, t)
+    pq = dev(torch.tensor([0.4, -0.9]))
+    held = {}
+    scratch = lambda name, shape, dt: held.setdefault((name, tuple(shape), dt), torch.empty(shape, dtype=dt, device="cuda"))
+    for with_scratch in (False, True):
+        fused = torch.empty(M, N, dtype=t, device="cuda")
+        o.take_launches()
+        o.gemm(a, w, fused, act=(o.ACT_XIELU, pq), scratch=scratch if with_scratch else None)
+        ran = o.take_launches()
+        assert "act.xielu" not in ran
+        pre = torch.empty(M, N, dtype=torch.float32, device="cuda")
+        o.gemm(a, w, pre, scratch=scratch if with_scratch else None)
+        apart = torch.empty(M, N, dtype=t, device="cuda")
+        o.act_xielu(pre, pq, apart)
+        assert torch.equal(fused, apart), sorted(ran)
+        want = plain.xielu(a.double().cpu() @ w.double().cpu().T, pq[0].double().cpu(), pq[1].double().cpu())
+        close(fused, want, 1e-5 if dtype == "f32" else 1e-2)
+    with pytest.raises(o.KernelError):
+        o.gemm(a, w, torch.zeros(M, N, dtype=torch.float32, device="cuda"), o.EPI_ADD, act=(o.ACT_XIELU, pq))
+
+
 @pytest.mark.parametrize("W", [1, 40, 131])
 def test_gated_recurrence_rows_state_and_slots(W):
     """Three requests of 1, 2 and 19 rows in one launch, states read from one slot and written to another; then each
