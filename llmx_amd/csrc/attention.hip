@@ -9,6 +9,7 @@
 // (the value product on the matrix cores reads several keys of one dim at a time).
 
 enum : int { QKNORM_NONE = 0, QKNORM_PROJECTION = 1, QKNORM_HEAD = 2 };
+#define ATT_PREP_MAX_D 256
 
 struct QkvArgs {
     const float* qkv;  // [T, q_width + 2 kv_width] f32: q | k | v
@@ -253,10 +254,113 @@ extern "C" int llmx_qknorm_rope_kvwrite(const float* qkv, const float* q_weight,
 }
 
 // ---------------------------------------------------------------------------
+// The same step for heads that are normed one by one: one wave a (row, head).  The projections' biases (optional) are added
+// first; each q and k head is then RMS-normed over its head_dim values with a weight of head_dim values shared by all
+// heads (norm_mode QKNORM_HEAD; QKNORM_NONE: no norm), its first rotary_dim dims are rotated, and k and v go to the row's
+// page.  Values have a width of their own (v_dim) and are not normed or rotated.  The row is q (H*D) | k (G*D) | v (G*VD).
+struct HeadPrepArgs {
+    const float* qkv;
+    const float* bias;       // [H*D + G*D + G*VD] or null
+    const float* q_weight;   // [D]
+    const float* k_weight;   // [D]
+    const float* cos_sin;
+    const int* pos;
+    const int* row_entry;
+    const int* tables;
+    void* q_out;
+    void* k_cache;           // [page][kv_head][token][D]
+    void* v_cache;           // [page][kv_head][VD][token]
+    float eps;
+    int n_heads, n_kv_heads, head_dim, v_dim, rotary_dim, norm_mode;
+    int page_tokens, max_blocks, write_kv, pairing;
+};
+
+template <typename T>
+__global__ void __launch_bounds__(64) head_norm_rope_kvwrite_kernel(HeadPrepArgs a) {
+    __shared__ float head[ATT_PREP_MAX_D];
+    const int t = blockIdx.x, hh = blockIdx.y, lane = threadIdx.x;
+    const int D = a.head_dim, VD = a.v_dim, H = a.n_heads, G = a.n_kv_heads;
+    const int width = H * D + G * D + G * VD;
+    const bool is_q = hh < H;
+    if (!is_q && !a.write_kv) return;
+    const int g = hh - H;
+    const int col0 = is_q ? hh * D : H * D + g * D;
+    const float* row = a.qkv + (size_t)t * width;
+    const int p = a.pos[t];
+    float x[ATT_PREP_MAX_D / 64];
+    float ss = 0.0f;
+#pragma unroll
+    for (int i = 0; i < ATT_PREP_MAX_D / 64; ++i) {
+        const int d = lane + 64 * i;
+        x[i] = d < D ? row[col0 + d] + (a.bias ? a.bias[col0 + d] : 0.0f) : 0.0f;
+        ss = fmaf(x[i], x[i], ss);
+    }
+    if (a.norm_mode == QKNORM_HEAD) {
+        const float r = 1.0f / sqrtf(wave_sum(ss) / (float)D + a.eps);
+        const float* w = is_q ? a.q_weight : a.k_weight;
+#pragma unroll
+        for (int i = 0; i < ATT_PREP_MAX_D / 64; ++i) {
+            const int d = lane + 64 * i;
+            if (d < D) x[i] = x[i] * (r * w[d]);
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < ATT_PREP_MAX_D / 64; ++i)
+        if (lane + 64 * i < D) head[lane + 64 * i] = x[i];
+    __syncthreads();
+    const float* cs = a.cos_sin + (size_t)p * a.rotary_dim;
+    const int half = a.rotary_dim / 2;
+    int page = 0, slot = 0;
+    if (!is_q) {
+        page = a.tables[(size_t)a.row_entry[t] * a.max_blocks + p / a.page_tokens];
+        slot = p % a.page_tokens;
+    }
+    const size_t head_at = (size_t)page * G + g;
+#pragma unroll
+    for (int i = 0; i < ATT_PREP_MAX_D / 64; ++i) {
+        const int d = lane + 64 * i;
+        if (d >= D) continue;
+        float y = x[i];
+        if (d < a.rotary_dim) {
+            const bool first = a.pairing == ROPE_HALVES ? d < half : (d & 1) == 0;
+            const int pair = a.pairing == ROPE_HALVES ? (first ? d : d - half) : d >> 1;
+            const float other = head[a.pairing == ROPE_HALVES ? (first ? d + half : d - half) : (first ? d + 1 : d - 1)];
+            const float c = cs[pair], sn = cs[half + pair];
+            y = first ? fmaf(-other, sn, y * c) : fmaf(other, sn, y * c);
+        }
+        if (is_q) st((T*)a.q_out + (size_t)t * H * D + col0 + d, y);
+        else st((T*)a.k_cache + (head_at * a.page_tokens + slot) * D + d, y);
+    }
+    if (!is_q) {
+        const int vcol = H * D + G * D + g * VD;
+        for (int d = lane; d < VD; d += 64)
+            st((T*)a.v_cache + (head_at * VD + d) * a.page_tokens + slot, row[vcol + d] + (a.bias ? a.bias[vcol + d] : 0.0f));
+    }
+}
+
+extern "C" int llmx_head_norm_rope_kvwrite(const float* qkv, const float* bias, const float* q_weight, const float* k_weight, const float* cos_sin,
+                                           const int* pos, const int* row_entry, const int* tables, void* q_out, void* k_cache, void* v_cache,
+                                           int dtype, float eps, int rows, int n_heads, int n_kv_heads, int head_dim, int v_dim, int rotary_dim,
+                                           int norm_mode, int page_tokens, int max_blocks, int write_kv, int pairing, hipStream_t stream) {
+    if (rows <= 0) return 0;
+    if (norm_mode != QKNORM_NONE && norm_mode != QKNORM_HEAD) return -2;
+    if (pairing != ROPE_HALVES && pairing != ROPE_INTERLEAVED) return -2;
+    if (head_dim < 1 || head_dim > ATT_PREP_MAX_D || v_dim < 1 || rotary_dim > head_dim || rotary_dim % 2) return -2;
+    if (norm_mode == QKNORM_HEAD && (!q_weight || !k_weight)) return -2;
+    HeadPrepArgs a{qkv, bias, q_weight, k_weight, cos_sin, pos, row_entry, tables, q_out, k_cache, v_cache, eps,
+                   n_heads, n_kv_heads, head_dim, v_dim, rotary_dim, norm_mode, page_tokens, max_blocks, write_kv, pairing};
+    llmx_note_launch(LK_HEAD_NORM_ROPE_KVWRITE);
+    const dim3 grid(rows, n_heads + n_kv_heads);
+    if (dtype == LLMX_F32) hipLaunchKernelGGL(head_norm_rope_kvwrite_kernel<float>, grid, dim3(64), 0, stream, a);
+    else hipLaunchKernelGGL(head_norm_rope_kvwrite_kernel<bf16_t>, grid, dim3(64), 0, stream, a);
+    return LLMX_CHECK_LAUNCH();
+}
+
+// ---------------------------------------------------------------------------
 // Universal paged attention: one wave per (row, head).  Keys lo..p of the row's request are walked in tiles of 64 in
 // position order with an online softmax; lo = max(0, p - window + 1) under a window, else 0.  Lane j of a tile owns key
 // lo + 64*tile + j for the scores; for the value sum lane d owns dims d, d+64, ... and walks the tile's keys in order.
-// A row's arithmetic depends on its own position and request only.
+// A row's arithmetic depends on its own position and request only.  Values may have a width of their own (v_dim).
 struct AttnArgs {
     const void* q;  // [T, n_heads, head_dim]
     const void* k_cache;
@@ -267,6 +371,7 @@ struct AttnArgs {
     void* out;  // [T, n_heads * head_dim]
     float scale;
     int n_heads, n_kv_heads, head_dim, page_tokens, max_blocks, window;
+    int v_dim;   // width of a value head (the output's too); keys and queries have head_dim
 };
 
 #define ATT_MAX_D 256
@@ -278,7 +383,7 @@ __global__ void __launch_bounds__(64) paged_attention_generic_kernel(AttnArgs a)
     __shared__ int heads_at[64];  // page * kv_heads + kv_head of each key of the tile
     __shared__ int slots[64];     // its place in the page
     const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
-    const int D = a.head_dim;
+    const int D = a.head_dim, VD = a.v_dim;
     const int kvh = h / (a.n_heads / a.n_kv_heads);
     const int p = a.pos[t];
     const int* table = a.tables + (size_t)a.row_entry[t] * a.max_blocks;
@@ -323,29 +428,29 @@ __global__ void __launch_bounds__(64) paged_attention_generic_kernel(AttnArgs a)
 #pragma unroll
         for (int i = 0; i < ATT_MAX_D / 64; ++i) {
             const int d = lane + 64 * i;
-            if (d < D) {
+            if (d < VD) {
                 float v = acc[i] * correction;
-                for (int jj = 0; jj < n; ++jj) v = fmaf(ps[jj], ld(vc + ((size_t)heads_at[jj] * D + d) * a.page_tokens + slots[jj]), v);
+                for (int jj = 0; jj < n; ++jj) v = fmaf(ps[jj], ld(vc + ((size_t)heads_at[jj] * VD + d) * a.page_tokens + slots[jj]), v);
                 acc[i] = v;
             }
         }
         m = m_new;
         __syncthreads();
     }
-    T* out = (T*)a.out + ((size_t)t * a.n_heads + h) * D;
+    T* out = (T*)a.out + ((size_t)t * a.n_heads + h) * VD;
 #pragma unroll
     for (int i = 0; i < ATT_MAX_D / 64; ++i) {
         const int d = lane + 64 * i;
-        if (d < D) st(out + d, acc[i] / l);
+        if (d < VD) st(out + d, acc[i] / l);
     }
 }
 
 extern "C" int llmx_paged_attention_generic(const void* q, const void* k_cache, const void* v_cache, const int* pos, const int* row_entry,
                                             const int* tables, void* out, int dtype, float scale, int rows, int n_heads, int n_kv_heads,
-                                            int head_dim, int page_tokens, int max_blocks, int window, hipStream_t stream) {
+                                            int head_dim, int page_tokens, int max_blocks, int window, int v_dim, hipStream_t stream) {
     if (rows <= 0) return 0;
-    if (head_dim > ATT_MAX_D || n_heads % n_kv_heads) return -2;
-    AttnArgs a{q, k_cache, v_cache, pos, row_entry, tables, out, scale, n_heads, n_kv_heads, head_dim, page_tokens, max_blocks, window};
+    if (head_dim > ATT_MAX_D || v_dim > ATT_MAX_D || v_dim < 1 || n_heads % n_kv_heads) return -2;
+    AttnArgs a{q, k_cache, v_cache, pos, row_entry, tables, out, scale, n_heads, n_kv_heads, head_dim, page_tokens, max_blocks, window, v_dim};
     llmx_note_launch(LK_ATTENTION_GENERIC);
     if (dtype == LLMX_F32)
         hipLaunchKernelGGL(paged_attention_generic_kernel<float>, dim3(rows, n_heads), dim3(64), 0, stream, a);

@@ -1,0 +1,277 @@
+// Mixers that carry a matrix state from token to token: for every head a float32 matrix S [D key channels, V value
+// channels] in the request's state slot, updated once a token:
+//     S <- diag(g_t) S                         (a decay a key channel, acting on S's rows)
+//     u  = beta_t (v_t - S^T k_t)              (delta rule; without it u = v_t: gated linear attention)
+//     S <- S + k_t u^T,   o_t = S^T q_t        (the read-out sees the token's own write)
+// A column of S (one value channel) never meets another, so the scan gives every column to four lanes that hold a quarter
+// of its D values each in registers and walk a request's rows in order: the state after a row is the same bits however
+// the rows were cut into steps.  Decays, gates, unit norms and the state are float32 in both number formats.
+// Around it: the preparation of a delta-rule row (short causal convolutions with silu, unit-norm q and k, the decay and
+// beta), the decay of gated linear attention, and the gated RMS norm of the read-out.
+#include "common.h"
+
+__device__ __forceinline__ float sigmoid_ls(float v) { return 1.0f / (1.0f + expf(-v)); }
+
+// ---------------------------------------------------------------------------
+// One block a row.  The fused in-projection's row `pre` holds q (G*D) | k (G*D) | v (H*V) at its start and beta's H
+// pre-activations at `beta_col`.  Channel c of q | k | v passes a causal convolution over the request's last `taps`
+// inputs (weights [C, taps], the last column weighs the row itself): inputs of earlier steps come from the tail the state
+// slot keeps ([taps - 1, C] at `tail_off`, oldest first; zero when the request opened), inputs of this step from `pre`.
+// Then silu; q and k heads are divided by sqrt(sum of squares + 1e-6); decay = exp(-exp(A_log[h]) softplus(step + dt_bias)).
+struct DeltaPrepArgs {
+    const float* pre;
+    int ld;
+    const float* conv_w;
+    const float* step_pre;   // [T, H*D]: the decay's projection before its bias
+    const float* dt_bias;    // [H*D]
+    const float* a_log;      // [H]
+    const float* state;
+    long state_stride;
+    int tail_off;
+    const int* slot_read;
+    const int* row_entry;
+    const int* entry_rows;
+    float* q;       // [T, G*D]
+    float* k;       // [T, G*D]
+    float* v;       // [T, H*V]
+    float* decay;   // [T, H*D]
+    float* beta;    // [T, H]
+    int G, H, D, V, taps, beta_col;
+};
+
+__global__ void __launch_bounds__(256) delta_prep_kernel(DeltaPrepArgs a) {
+    extern __shared__ float chan[];
+    const int t = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int GD = a.G * a.D, HV = a.H * a.V, HD = a.H * a.D;
+    const int C = 2 * GD + HV;
+    const int e = a.row_entry[t];
+    const int row0 = a.entry_rows[2 * e];
+    const int i = t - row0;
+    const float* tail = a.state + (size_t)a.slot_read[e] * a.state_stride + a.tail_off;
+    for (int c = tid; c < C; c += 256) {
+        float acc = 0.0f;
+        for (int j = 0; j < a.taps; ++j) {
+            const int idx = i - (a.taps - 1) + j;
+            const float x = idx >= 0 ? a.pre[(size_t)(row0 + idx) * a.ld + c] : tail[(size_t)(a.taps - 1 + idx) * C + c];
+            acc = fmaf(a.conv_w[(size_t)c * a.taps + j], x, acc);
+        }
+        chan[c] = acc * sigmoid_ls(acc);
+    }
+    __syncthreads();
+    for (int hh = wave; hh < 2 * a.G; hh += 4) {
+        const float* head = chan + (size_t)hh * a.D;
+        float ss = 0.0f;
+        for (int d = lane; d < a.D; d += 64) ss = fmaf(head[d], head[d], ss);
+        const float r = 1.0f / sqrtf(wave_sum(ss) + 1e-6f);
+        float* out = (hh < a.G ? a.q + (size_t)t * GD + (size_t)hh * a.D : a.k + (size_t)t * GD + (size_t)(hh - a.G) * a.D);
+        for (int d = lane; d < a.D; d += 64) out[d] = head[d] * r;
+    }
+    for (int c = tid; c < HV; c += 256) a.v[(size_t)t * HV + c] = chan[2 * GD + c];
+    for (int c = tid; c < HD; c += 256) {
+        const float sp = softplus_f(a.step_pre[(size_t)t * HD + c] + a.dt_bias[c]);
+        a.decay[(size_t)t * HD + c] = expf(-expf(a.a_log[c / a.D]) * sp);
+    }
+    for (int c = tid; c < a.H; c += 256) a.beta[(size_t)t * a.H + c] = sigmoid_ls(a.pre[(size_t)t * a.ld + a.beta_col + c]);
+}
+
+extern "C" int llmx_delta_prep(const float* pre, int ld, const float* conv_w, const float* step_pre, const float* dt_bias, const float* a_log,
+                               const float* state, long state_stride, int tail_off, const int* slot_read, const int* row_entry,
+                               const int* entry_rows, float* q, float* k, float* v, float* decay, float* beta, int rows, int G, int H, int D, int V,
+                               int taps, int beta_col, hipStream_t stream) {
+    if (rows <= 0) return 0;
+    const long C = 2L * G * D + (long)H * V;
+    if (taps < 1 || G < 1 || H % G || C * (long)sizeof(float) > 64 * 1024 || beta_col + H > ld || C > ld) return -2;
+    DeltaPrepArgs a{pre, ld, conv_w, step_pre, dt_bias, a_log, state, state_stride, tail_off, slot_read, row_entry, entry_rows,
+                    q, k, v, decay, beta, G, H, D, V, taps, beta_col};
+    llmx_note_launch(LK_DELTA_PREP);
+    hipLaunchKernelGGL(delta_prep_kernel, dim3(rows), dim3(256), (size_t)C * sizeof(float), stream, a);
+    return LLMX_CHECK_LAUNCH();
+}
+
+// ---------------------------------------------------------------------------
+// The decay of gated linear attention: out = sigmoid(z + b)^(1 / tau) = exp(-softplus(-(z + b)) / tau), element by element.
+__global__ void __launch_bounds__(256) sigmoid_root_kernel(const float* __restrict__ z, const float* __restrict__ bias, float inv_tau,
+                                                         float* __restrict__ out, int n, size_t total) {
+    const size_t at = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (at >= total) return;
+    const float x = z[at] + (bias ? bias[(int)(at % (size_t)n)] : 0.0f);
+    out[at] = expf(-softplus_f(-x) * inv_tau);
+}
+
+extern "C" int llmx_sigmoid_root(const float* z, const float* bias, float inv_tau, float* out, int rows, int n, hipStream_t stream) {
+    if (rows <= 0 || n <= 0) return 0;
+    llmx_note_launch(LK_SIGMOID_ROOT);
+    const size_t total = (size_t)rows * n;
+    hipLaunchKernelGGL(sigmoid_root_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, z, bias, inv_tau, out, n, total);
+    return LLMX_CHECK_LAUNCH();
+}
+
+// ---------------------------------------------------------------------------
+// The scan.  Grid (H * ceil(V / 16), entries), one wave a block: lane = 16 s + c owns value channel 16 * tile + c and
+// key channels [s R, s R + R) of its head.  q and k are read head h / share (several heads may share one), with row
+// strides of their own, so they may be columns of a wider projection.  The next row's operands are asked for before this
+// row is worked on.  Sums over a column's four lanes: (s0 + s1) + (s2 + s3).
+// The block of tile 0 of an entry also hands on the convolution tail: the entry's last taps - 1 inputs, from this step's
+// rows of `tail_src` and, where the step brought fewer, from the old tail.
+struct StateScanArgs {
+    const float* q;
+    const float* k;
+    const float* v;
+    const float* decay;
+    const float* beta;   // [T, H] or null: no delta correction
+    int ldq, ldk, ldv, ldg;
+    float* state;
+    long state_stride;
+    const int* slot_read;
+    const int* slot_write;
+    const int* entry_rows;
+    float* out;          // [T, H*V]
+    float out_scale;
+    int H, share, D, V;
+    const float* tail_src;
+    int tail_ld, tail_C, taps, tail_off;
+};
+
+template <int R, bool AHEAD>
+__global__ void __launch_bounds__(64) state_scan_kernel(StateScanArgs a) {
+    const int lane = threadIdx.x, s = lane >> 4, c = lane & 15;
+    const int tiles = (a.V + 15) / 16;
+    const int h = blockIdx.x / tiles, tile = blockIdx.x % tiles;
+    const int e = blockIdx.y;
+    const int row0 = a.entry_rows[2 * e], n = a.entry_rows[2 * e + 1];
+    const int j = tile * 16 + c;
+    const bool col = j < a.V;
+    const int d0 = s * R;
+    const size_t slot_r = (size_t)a.slot_read[e] * a.state_stride, slot_w = (size_t)a.slot_write[e] * a.state_stride;
+
+    if (a.taps > 1 && blockIdx.x == 0) {
+        const float* old = a.state + slot_r + a.tail_off;
+        float* fresh = a.state + slot_w + a.tail_off;
+        for (int ch = lane; ch < a.tail_C; ch += 64) {
+            for (int p = 0; p < a.taps - 1; ++p) {      // ascending: in place, a value is read before its place is written
+                const int idx = n - (a.taps - 1) + p;
+                fresh[(size_t)p * a.tail_C + ch] = idx >= 0 ? a.tail_src[(size_t)(row0 + idx) * a.tail_ld + ch] : old[(size_t)(n + p) * a.tail_C + ch];
+            }
+        }
+    }
+
+    float S[R];
+    {
+        const float* src = a.state + slot_r + ((size_t)h * a.D) * a.V + j;
+#pragma unroll
+        for (int i = 0; i < R; ++i) S[i] = (col && d0 + i < a.D) ? src[(size_t)(d0 + i) * a.V] : 0.0f;
+    }
+    const int hq = h / a.share;
+    const float* qp = a.q + (size_t)hq * a.D;
+    const float* kp = a.k + (size_t)hq * a.D;
+    const float* gp = a.decay + (size_t)h * a.D;
+    const float* vp = a.v + (size_t)h * a.V + (col ? j : 0);
+    float nk[R], nq[R], ng[R], nv, nb = 0.0f;
+    auto fetch = [&](int t) {
+        const size_t row = (size_t)(row0 + t);
+#pragma unroll
+        for (int i = 0; i < R; ++i) {
+            const bool in = d0 + i < a.D;
+            const int d = in ? d0 + i : 0;
+            const float kv = kp[row * a.ldk + d], qv = qp[row * a.ldq + d], gv = gp[row * a.ldg + d];
+            nk[i] = in ? kv : 0.0f;
+            nq[i] = in ? qv : 0.0f;
+            ng[i] = in ? gv : 0.0f;
+        }
+        nv = vp[row * a.ldv];
+        if (a.beta) nb = a.beta[row * a.H + h];
+    };
+    if (AHEAD) fetch(0);
+    for (int t = 0; t < n; ++t) {
+        if (!AHEAD) fetch(t);      // a quarter column of 64 values leaves no registers for a second set of operands
+        float ck[R], cq[R], cg[R];
+#pragma unroll
+        for (int i = 0; i < R; ++i) {
+            ck[i] = nk[i];
+            cq[i] = nq[i];
+            cg[i] = ng[i];
+        }
+        const float cv = nv, cb = nb;
+        if (AHEAD) fetch(t + 1 < n ? t + 1 : n - 1);
+        float u = cv;
+        if (a.beta) {
+            float p = 0.0f;
+#pragma unroll
+            for (int i = 0; i < R; ++i) {
+                S[i] = S[i] * cg[i];
+                p = fmaf(ck[i], S[i], p);
+            }
+            u = cb * (cv - rows_sum4(p));
+        } else {
+#pragma unroll
+            for (int i = 0; i < R; ++i) S[i] = S[i] * cg[i];
+        }
+        float o = 0.0f;
+#pragma unroll
+        for (int i = 0; i < R; ++i) {
+            S[i] = fmaf(ck[i], u, S[i]);
+            o = fmaf(cq[i], S[i], o);
+        }
+        o = rows_sum4(o);
+        if (s == 0 && col) a.out[(size_t)(row0 + t) * a.H * a.V + (size_t)h * a.V + j] = o * a.out_scale;
+    }
+    {
+        float* dst = a.state + slot_w + ((size_t)h * a.D) * a.V + j;
+#pragma unroll
+        for (int i = 0; i < R; ++i)
+            if (col && d0 + i < a.D) dst[(size_t)(d0 + i) * a.V] = S[i];
+    }
+}
+
+extern "C" int llmx_state_scan(const float* q, int ldq, const float* k, int ldk, const float* v, int ldv, const float* decay, int ldg,
+                               const float* beta, float* state, long state_stride, const int* slot_read, const int* slot_write,
+                               const int* entry_rows, float* out, float out_scale, int n_entries, int H, int share, int D, int V,
+                               const float* tail_src, int tail_ld, int tail_C, int taps, int tail_off, hipStream_t stream) {
+    if (n_entries <= 0) return 0;
+    if (H < 1 || share < 1 || H % share || D < 1 || D > 256 || V < 1 || (taps > 1 && !tail_src)) return -2;
+    StateScanArgs a{q, k, v, decay, beta, ldq, ldk, ldv, ldg, state, state_stride, slot_read, slot_write, entry_rows, out, out_scale,
+                    H, share, D, V, tail_src, tail_ld, tail_C, taps, tail_off};
+    const dim3 grid((unsigned)(H * ((V + 15) / 16)), (unsigned)n_entries);
+    llmx_note_launch(LK_STATE_SCAN);
+    const int per_lane = (D + 3) / 4;
+    if (per_lane <= 8) hipLaunchKernelGGL((state_scan_kernel<8, true>), grid, dim3(64), 0, stream, a);
+    else if (per_lane <= 16) hipLaunchKernelGGL((state_scan_kernel<16, true>), grid, dim3(64), 0, stream, a);
+    else if (per_lane <= 32) hipLaunchKernelGGL((state_scan_kernel<32, true>), grid, dim3(64), 0, stream, a);
+    else hipLaunchKernelGGL((state_scan_kernel<64, false>), grid, dim3(64), 0, stream, a);
+    return LLMX_CHECK_LAUNCH();
+}
+
+// ---------------------------------------------------------------------------
+// The read-out's gated norm, one wave a (row, head): out = o / sqrt(mean(o^2) + eps) * w * gate(z), gate = sigmoid or silu
+// of the gate's pre-activation z (a float32 view with its own row stride); out in the activation type for the output
+// projection.
+enum : int { GATE_SIGMOID = 0, GATE_SILU = 1 };
+
+template <typename TO>
+__global__ void __launch_bounds__(64) head_norm_gate_kernel(const float* __restrict__ o, const float* __restrict__ w, const float* __restrict__ z,
+                                                          int ldz, TO* __restrict__ out, float eps, int H, int V, int gate) {
+    const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+    const float* row = o + ((size_t)t * H + h) * V;
+    float ss = 0.0f;
+    for (int j = lane; j < V; j += 64) ss = fmaf(row[j], row[j], ss);
+    const float r = 1.0f / sqrtf(wave_sum(ss) / (float)V + eps);
+    const float* zr = z + (size_t)t * ldz + (size_t)h * V;
+    TO* dst = out + ((size_t)t * H + h) * V;
+    for (int j = lane; j < V; j += 64) {
+        const float x = zr[j];
+        const float g = gate == GATE_SIGMOID ? sigmoid_ls(x) : x * sigmoid_ls(x);
+        st(dst + j, row[j] * r * w[j] * g);
+    }
+}
+
+extern "C" int llmx_head_norm_gate(const float* o, const float* w, const float* z, int ldz, void* out, int out_dtype, float eps, int rows, int H,
+                                   int V, int gate, hipStream_t stream) {
+    if (rows <= 0) return 0;
+    if (H < 1 || V < 1 || (gate != GATE_SIGMOID && gate != GATE_SILU)) return -2;
+    llmx_note_launch(LK_HEAD_NORM_GATE);
+    if (out_dtype == LLMX_F32)
+        hipLaunchKernelGGL(head_norm_gate_kernel<float>, dim3(rows, H), dim3(64), 0, stream, o, w, z, ldz, (float*)out, eps, H, V, gate);
+    else
+        hipLaunchKernelGGL(head_norm_gate_kernel<bf16_t>, dim3(rows, H), dim3(64), 0, stream, o, w, z, ldz, (bf16_t*)out, eps, H, V, gate);
+    return LLMX_CHECK_LAUNCH();
+}

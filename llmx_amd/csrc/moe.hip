@@ -98,18 +98,20 @@ __device__ __forceinline__ void route_row_256(const float (&x)[4], const float (
 // the largest key not yet taken is picked, the lowest id on ties; the weight is the unbiased s_e, divided by the
 // picks' sum (added in pick order) when `normalize`, then times `scale`.  A row with a non-finite key gets ids -1 and
 // weights 0.  Ids and weights come out in pick order, best first.
+// `logit_bias` (optional): added to the logits (and kept in z) before anything else: a router whose bias is part of its
+// logits, so that scores and weights see it too.
 // `parts` (optional): the logits arrive as `slices` partial sums [slices][rows][experts]; the row adds them in slice order
 // into z first.
 __global__ void __launch_bounds__(64) route_topk_kernel(float* __restrict__ z, const float* __restrict__ parts, int slices, long slice_stride,
                                                        const float* __restrict__ bias, int* __restrict__ ids,
                                                        float* __restrict__ weights, int n_experts, int k, int score, int normalize,
-                                                       float scale) {
+                                                       float scale, const float* __restrict__ logit_bias) {
     __shared__ float s[ROUTE_MAX_EXPERTS];
     __shared__ float b[ROUTE_MAX_EXPERTS];
     __shared__ float chosen[ROUTE_MAX_K];
     const int r = blockIdx.x, lane = threadIdx.x;
     float* row = z + (size_t)r * n_experts;
-    if (score == SCORE_SIGMOID && n_experts <= 256 && k <= 64) {   // the row fits the wave's registers
+    if (score == SCORE_SIGMOID && n_experts <= 256 && k <= 64 && !logit_bias) {   // the row fits the wave's registers
         float x[4], bias_v[4], weight;
         int id;
         load_row_256(row, parts ? parts + (size_t)r * n_experts : nullptr, slices, slice_stride, bias, n_experts, lane, x, bias_v);
@@ -124,6 +126,9 @@ __global__ void __launch_bounds__(64) route_topk_kernel(float* __restrict__ z, c
         for (int e = lane; e < n_experts; e += 64) {   // the thread reads back only what it wrote
             row[e] = sum_slices(parts + (size_t)r * n_experts + e, slices, slice_stride);
         }
+    }
+    if (logit_bias) {   // a bias that belongs to the logits themselves: it moves the scores, not only the pick keys
+        for (int e = lane; e < n_experts; e += 64) row[e] = row[e] + logit_bias[e];
     }
     float row_max = -INFINITY;
     if (score == SCORE_SOFTMAX) {
@@ -187,12 +192,13 @@ __global__ void __launch_bounds__(64) route_topk_kernel(float* __restrict__ z, c
 }
 
 extern "C" int llmx_route_topk(float* z, const float* parts, int slices, long slice_stride, const float* bias, int* ids, float* weights,
-                               int rows, int n_experts, int k, int score, int normalize, float scale, hipStream_t stream) {
+                               int rows, int n_experts, int k, int score, int normalize, float scale, const float* logit_bias,
+                               hipStream_t stream) {
     if (rows <= 0) return 0;
     if (n_experts > ROUTE_MAX_EXPERTS || k > ROUTE_MAX_K || k > n_experts || k <= 0 || (parts && (slices < 1 || slices > ROUTE_MAX_SLICES))) return -2;
     llmx_note_launch(LK_ROUTE_TOPK);
     hipLaunchKernelGGL(route_topk_kernel, dim3(rows), dim3(64), 0, stream, z, parts, slices, slice_stride, bias, ids, weights, n_experts, k, score,
-                       normalize, scale);
+                       normalize, scale, logit_bias);
     return LLMX_CHECK_LAUNCH();
 }
 

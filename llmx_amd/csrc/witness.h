@@ -62,7 +62,17 @@
     X(LATENT_ATTENTION_TILES, "latent_attention.tiles")                                                                   \
     X(LATENT_ATTENTION_ROWS, "latent_attention.rows")                                                                     \
     X(LATENT_ATTENTION_MERGE, "latent_attention.merge")                                                                   \
-    X(HEAD_GATE, "head_gate")
+    X(HEAD_GATE, "head_gate")                                                                                             \
+    X(LAYERNORM, "layernorm")                                                                                             \
+    X(LAYERNORM_ADD, "layernorm_add")                                                                                     \
+    X(CAST_ROWS, "cast_rows")                                                                                             \
+    X(COMBINE_ROWS, "combine_rows")                                                                                       \
+    X(SCALE_SOFTCAP, "scale_softcap")                                                                                     \
+    X(HEAD_NORM_ROPE_KVWRITE, "head_norm_rope_kvwrite")                                                                   \
+    X(DELTA_PREP, "delta_prep")                                                                                           \
+    X(SIGMOID_ROOT, "sigmoid_root")                                                                                       \
+    X(STATE_SCAN, "state_scan")                                                                                           \
+    X(HEAD_NORM_GATE, "head_norm_gate")
 
 enum LlmxLaunchKind : int {
 #define LLMX_X(id, name) LK_##id,

@@ -19,7 +19,7 @@ from .. import ops
 from ..cache import CacheManager, GroupSpec, OutOfPages
 from ..models import registry
 from ..parts.base import BuildContext, LayerCache, Part
-from ..parts.spec import ModelSpec, PagedNeed, StateNeed
+from ..parts.spec import CompositeNeed, ModelSpec, PagedNeed, StateNeed
 from ..weights import ModelFiles, RandomInit, load as load_weights
 from ..weights.loader import device_dtype
 from ..weights.random_init import fill_random, stored_dtype
@@ -145,56 +145,75 @@ class Engine:
 
     def _make_cache(self) -> None:
         """Allocates what the mixers' needs list: for every group of equal paged needs a page pool and, for each of the
-        need's tensors, one arena [caches of the group, pages, *page shape]; for every state need [slots, *shape]."""
+        need's tensors, one arena [caches of the group, pages, *page shape]; for every state need [slots, *shape].  A
+        composite need's members are treated one by one, each as a mixer's own need would be."""
         needs = self.model.cache_needs()
         n_pages = self.kv_tokens // self.page_tokens
+        # the needs' leaves in run-order numbering: (cache number, path of member indices, need)
+        leaves = []
+
+        def walk(number, path, need):
+            if isinstance(need, CompositeNeed):
+                for i, m in enumerate(need.members):
+                    walk(number, path + (i,), m)
+            else:
+                leaves.append((number, path, need))
+
+        for number, need in enumerate(needs):
+            walk(number, (), need)
         keys: List[PagedNeed] = []
-        self._group_of: List[int] = []          # cache number -> group (or -1)
-        self._index_in_group: List[int] = []
         counts: List[int] = []
-        for need in needs:
+        place = {}                              # (cache number, path) -> (group, index in group) of a paged leaf
+        for number, path, need in leaves:
             if isinstance(need, PagedNeed):
                 if need not in keys:
                     keys.append(need)
                     counts.append(0)
                 g = keys.index(need)
-                self._group_of.append(g)
-                self._index_in_group.append(counts[g])
+                place[(number, path)] = (g, counts[g])
                 counts[g] += 1
-            else:
-                self._group_of.append(-1)
-                self._index_in_group.append(-1)
+        self._group_of = [place.get((i, ()), (-1, -1))[0] for i in range(len(needs))]          # cache number -> group (or -1)
+        self._index_in_group = [place.get((i, ()), (-1, -1))[1] for i in range(len(needs))]
         self.group_needs = keys
         groups = [GroupSpec(f"kv{g}", self.page_tokens, n_pages, need.window) for g, need in enumerate(keys)]
         groups = [replace(g, n_pages=g.pool_pages(self.kv_tokens, self.max_requests, self.step_tokens)) for g in groups]
         # a model with per-request state steps into a second slot, so that a step that fails leaves the state as it was
-        self._stateful = any(isinstance(need, StateNeed) for need in needs)
+        self._stateful = any(isinstance(need, StateNeed) for _, _, need in leaves)
         self.cache = CacheManager(groups, self.max_requests, shadow_slots=self._stateful)
         self._paged: List[Dict[str, torch.Tensor]] = []
         for g, need in enumerate(keys):
             self._paged.append({t.name: torch.zeros((counts[g], groups[g].n_pages, *t.page_shape(self.page_tokens)),
                                                     dtype=getattr(torch, t.dtype) if t.dtype else self.act_dtype, device=self.device)
                                 for t in need.tensors})
-        self._state: List[Optional[torch.Tensor]] = []
-        for need in needs:
-            if isinstance(need, StateNeed):
-                self._state.append(torch.zeros((self.cache.slots.capacity, *need.shape), dtype=getattr(torch, need.dtype), device=self.device))
-            else:
-                self._state.append(None)
         # which states a step must copy into its slot beforehand: those of mixers that step in place
         writers = {e.cache: self.model.blocks[e.layer].mixer for e in self.spec.run_order if e.writes}
-        self._state_copied = [isinstance(need, StateNeed) and not getattr(writers[i], "steps_between_slots", False)
-                              for i, need in enumerate(needs)]
+
+        def member_of(mixer, path):
+            for i in path:
+                mixer = mixer.members()[i]
+            return mixer
+
+        self._state: List[Optional[torch.Tensor]] = []
+        self._state_copied: List[bool] = []
+        state_at = {}
+        for number, path, need in leaves:
+            if isinstance(need, StateNeed):
+                state_at[(number, path)] = len(self._state)
+                self._state.append(torch.zeros((self.cache.slots.capacity, *need.shape), dtype=getattr(torch, need.dtype), device=self.device))
+                self._state_copied.append(not getattr(member_of(writers[number], path), "steps_between_slots", False))
         self._copy_state = any(self._state_copied)
-        self._layer_caches: List[LayerCache] = []
-        for e in self.spec.run_order:
-            g = self._group_of[e.cache]
-            if g >= 0:
-                at = self._index_in_group[e.cache]
-                self._layer_caches.append(LayerCache(group=g, tensors={name: arena[at] for name, arena in self._paged[g].items()},
-                                                     writes=e.writes))
-            else:
-                self._layer_caches.append(LayerCache(state=self._state[e.cache], writes=e.writes))
+
+        def cache_of(number, path, need, writes):
+            if isinstance(need, CompositeNeed):
+                return LayerCache(writes=writes, members=[cache_of(number, path + (i,), m, writes) for i, m in enumerate(need.members)])
+            if isinstance(need, PagedNeed):
+                g, at = place[(number, path)]
+                return LayerCache(group=g, tensors={name: arena[at] for name, arena in self._paged[g].items()}, writes=writes)
+            if isinstance(need, StateNeed):
+                return LayerCache(state=self._state[state_at[(number, path)]], writes=writes)
+            return LayerCache(writes=writes)
+
+        self._layer_caches: List[LayerCache] = [cache_of(e.cache, (), needs[e.cache], e.writes) for e in self.spec.run_order]
 
     # -- requests ---------------------------------------------------------------
     def add_request(self, request: Hashable) -> int:

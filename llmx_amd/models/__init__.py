@@ -4,6 +4,7 @@ from .registry import (ArchitectureEntry, architecture_of, architectures, assemb
                        register_architecture, unregister_architecture)
 from . import minimax_m3  # noqa: F401  (registers MiniMaxM3ForCausalLM)
 from . import nenotar  # noqa: F401  (registers Nenotar)
+from . import bonerax  # noqa: F401  (registers Bonerax)
 
 __all__ = ["ArchitectureEntry", "architecture_of", "architectures", "assemble", "read_config", "read_model_dir",
            "register_architecture", "unregister_architecture"]

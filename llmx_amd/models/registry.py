@@ -60,6 +60,13 @@ def read_config(values: dict):
 def read_model_dir(path: str | Path):
     """(configuration, ModelSpec) of the model folder `path` (config.json decides the class)."""
     cfg = read_config(read_json(Path(path) / "config.json"))
+    if hasattr(cfg, "with_tensor_shapes"):      # a design that leaves some sizes to its tensors' shapes
+        from ..weights import ModelFiles
+        files = ModelFiles(path)
+        try:
+            cfg = cfg.with_tensor_shapes({n: tuple(files.entry(n).shape) for n in files.names()})
+        finally:
+            files.close()
     return cfg, assemble(cfg)
 
 

@@ -74,9 +74,19 @@ def _declare(h) -> None:
         "llmx_attention_partial_pad": [],
         "llmx_gemm_generic": [P, I, P, I, P, I, I, I, I, I, I, I, I, I, P, P, I, L, I, I, P, P],
         "llmx_qknorm_rope_kvwrite": [P, P, P, P, P, P, P, P, P, P, I, F, I, I, I, I, I, I, I, I, I, I, P],
-        "llmx_paged_attention_generic": [P, P, P, P, P, P, P, I, F, I, I, I, I, I, I, I, P],
+        "llmx_paged_attention_generic": [P, P, P, P, P, P, P, I, F, I, I, I, I, I, I, I, I, P],
+        "llmx_head_norm_rope_kvwrite": [P, P, P, P, P, P, P, P, P, P, P, I, F, I, I, I, I, I, I, I, I, I, I, I, P],
+        "llmx_layernorm": [P, P, P, F, P, I, P, I, I, P],
+        "llmx_layernorm_add": [P, P, P, F, P, I, I, I, P],
+        "llmx_cast_rows": [P, P, I, L, P],
+        "llmx_combine_rows": [P, P, F, P, P, F, I, I, I, P],
+        "llmx_scale_softcap": [P, F, F, L, P],
+        "llmx_delta_prep": [P, I, P, P, P, P, P, L, I, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, P],
+        "llmx_sigmoid_root": [P, P, F, P, I, I, P],
+        "llmx_state_scan": [P, I, P, I, P, I, P, I, P, P, L, P, P, P, P, F, I, I, I, I, I, P, I, I, I, I, P],
+        "llmx_head_norm_gate": [P, P, P, I, P, I, F, I, I, I, I, P],
         "llmx_paged_attention_mfma": [P, P, P, P, P, P, P, I, I, I, P, I, P, P, P, F, I, I, I, I, I, I, I, P],
-        "llmx_route_topk": [P, P, I, L, P, P, P, I, I, I, I, I, F, P],
+        "llmx_route_topk": [P, P, I, L, P, P, P, I, I, I, I, I, F, P, P],
         "llmx_moe_align": [P, I, I, P, P, P, P, P, P, P, P],
         "llmx_route_topk_align": [P, P, I, L, P, P, P, I, I, I, I, F, P, P, P, P, P, P],
         "llmx_gemm_skinny": [P, P, P, I, I, I, I, I, I, I, I, I, I, P, P, P, P, I, L, I, P, P, F, I, I, P, P],
@@ -464,6 +474,139 @@ def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: Optional[tor
                               _dev(out32, "out32", torch.float32, (rows, n)), rows, n, _stream()), "rmsnorm")
 
 
+def layernorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: Optional[torch.Tensor], out32: Optional[torch.Tensor] = None,
+              pick: Optional[torch.Tensor] = None) -> None:
+    """out[r] = (x - mean) / sqrt(var + eps) * weight of row x[pick[r]] (or x[r]), var the mean of the squared deviations;
+    out in its own dtype, out32 an optional float32 copy."""
+    n = x.shape[-1]
+    rows = pick.shape[0] if pick is not None else x.shape[0]
+    if out is None and out32 is None:
+        raise KernelError("layernorm needs an output")
+    _check(lib().llmx_layernorm(_dev(x, "x", torch.float32), _dev(pick, "pick", torch.int32), _dev(weight, "weight", torch.float32, (n,)),
+                                float(eps), _dev(out, "out", shape=(rows, n)), _code(out.dtype) if out is not None else F32,
+                                _dev(out32, "out32", torch.float32, (rows, n)), rows, n, _stream()), "layernorm")
+
+
+def layernorm_add(x: torch.Tensor, y: torch.Tensor, weight: torch.Tensor, eps: float, copy: Optional[torch.Tensor] = None) -> None:
+    """x += layer norm of y (weight, no bias), float32 rows; `copy` receives the new rows in its type."""
+    rows, n = x.shape
+    _check(lib().llmx_layernorm_add(_dev(x, "x", torch.float32), _dev(y, "y", torch.float32, (rows, n)), _dev(weight, "weight", torch.float32, (n,)),
+                                    float(eps), _dev(copy, "copy", shape=(rows, n)), _code(copy.dtype) if copy is not None else F32, rows, n,
+                                    _stream()), "layernorm_add")
+
+
+def cast_rows(x: torch.Tensor, out: torch.Tensor) -> None:
+    """out = x (float32) in out's type."""
+    if out.shape != x.shape:
+        raise KernelError("cast_rows: shapes do not agree")
+    _check(lib().llmx_cast_rows(_dev(x, "x", torch.float32), _dev(out, "out"), _code(out.dtype), x.numel(), _stream()), "cast_rows")
+
+
+def combine_rows(out: torch.Tensor, a: torch.Tensor, scale_a: float = 1.0, bias_a: Optional[torch.Tensor] = None,
+                 b: Optional[torch.Tensor] = None, scale_b: float = 1.0, accumulate: bool = False) -> None:
+    """out (= or +=) scale_a * (a + bias_a) + scale_b * b over float32 rows [T, n]; bias_a [n] and b may be None."""
+    rows, n = out.shape
+    _check(lib().llmx_combine_rows(_dev(out, "out", torch.float32), _dev(a, "a", torch.float32, (rows, n)), float(scale_a),
+                                   _dev(bias_a, "bias_a", torch.float32, (n,)), _dev(b, "b", torch.float32, (rows, n)), float(scale_b),
+                                   1 if accumulate else 0, rows, n, _stream()), "combine_rows")
+
+
+def scale_softcap(z: torch.Tensor, scale: float, cap: float) -> None:
+    """z <- z * scale, then cap * tanh(z / cap) when cap > 0; float32, in place."""
+    _check(lib().llmx_scale_softcap(_dev(z, "z", torch.float32), float(scale), float(cap), z.numel(), _stream()), "scale_softcap")
+
+
+def _rows_view(t: torch.Tensor, name: str, rows: int, cols: int):
+    """(address, row stride) of a float32 [rows, cols] tensor whose rows may be columns of a wider one."""
+    if not isinstance(t, torch.Tensor) or not t.is_cuda or t.dtype != torch.float32 or tuple(t.shape) != (rows, cols) or (cols > 1 and t.stride(1) != 1):
+        raise KernelError(f"{name} must be float32 [{rows}, {cols}] on the GPU with unit stride along a row")
+    return t.data_ptr(), (t.stride(0) if rows > 1 else max(cols, t.stride(0)))
+
+
+def delta_prep(pre: torch.Tensor, conv_w: torch.Tensor, step_pre: torch.Tensor, dt_bias: torch.Tensor, a_log: torch.Tensor,
+               state: torch.Tensor, tail_off: int, slot_read: torch.Tensor, row_entry: torch.Tensor, entry_rows: torch.Tensor,
+               q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay: torch.Tensor, beta: torch.Tensor, G: int, H: int, D: int, V: int,
+               beta_col: int) -> None:
+    """A delta-rule mixer's rows made ready for the scan (see csrc/linear_state.hip): from the fused in-projection `pre`
+    [T, ld] = q (G*D) | k (G*D) | v (H*V) | ... | beta (H) at beta_col: the short causal convolution (conv_w [C, taps], the
+    inputs of earlier steps from the state's tail at `tail_off`) with silu, unit-norm q and k heads, v, the decay
+    exp(-exp(a_log) softplus(step_pre + dt_bias)) [T, H*D] and beta = sigmoid [T, H]."""
+    T, ld = pre.shape
+    C = 2 * G * D + H * V
+    taps = conv_w.shape[1]
+    n_e = entry_rows.shape[0]
+    if state.dim() != 2 or tail_off + (taps - 1) * C > state.shape[1]:
+        raise KernelError("delta_prep: the state does not hold the convolution's tail")
+    _check(lib().llmx_delta_prep(_dev(pre, "pre", torch.float32), ld, _dev(conv_w, "conv_w", torch.float32, (C, taps)),
+                                 _dev(step_pre, "step_pre", torch.float32, (T, H * D)), _dev(dt_bias, "dt_bias", torch.float32, (H * D,)),
+                                 _dev(a_log, "a_log", torch.float32, (H,)), _dev(state, "state", torch.float32), state.shape[1], int(tail_off),
+                                 _dev(slot_read, "slot_read", torch.int32, (n_e,)), _dev(row_entry, "row_entry", torch.int32, (T,)),
+                                 _dev(entry_rows, "entry_rows", torch.int32, (n_e, 2)), _dev(q, "q", torch.float32, (T, G * D)),
+                                 _dev(k, "k", torch.float32, (T, G * D)), _dev(v, "v", torch.float32, (T, H * V)),
+                                 _dev(decay, "decay", torch.float32, (T, H * D)), _dev(beta, "beta", torch.float32, (T, H)),
+                                 T, G, H, D, V, taps, int(beta_col), _stream()), "delta_prep")
+
+
+def sigmoid_root(z: torch.Tensor, bias: Optional[torch.Tensor], tau: float, out: torch.Tensor) -> None:
+    """out = sigmoid(z + bias)^(1 / tau), float32 [T, n]."""
+    rows, n = z.shape
+    _check(lib().llmx_sigmoid_root(_dev(z, "z", torch.float32), _dev(bias, "bias", torch.float32, (n,)), 1.0 / float(tau),
+                                   _dev(out, "out", torch.float32, (rows, n)), rows, n, _stream()), "sigmoid_root")
+
+
+def state_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay: torch.Tensor, beta: Optional[torch.Tensor], state: torch.Tensor,
+               slot_read: torch.Tensor, slot_write: torch.Tensor, entry_rows: torch.Tensor, out: torch.Tensor, out_scale: float,
+               H: int, qk_heads: int, D: int, V: int, tail=None) -> None:
+    """The matrix-state recurrence over each entry's rows (csrc/linear_state.hip): per head S <- diag(decay) S;
+    u = beta (v - S^T k) (u = v without beta); S <- S + k u^T; out = out_scale * S^T q.  q, k [T, qk_heads*D], v [T, H*V],
+    decay [T, H*D] are float32 views whose rows may be columns of wider tensors; state [slots, width] float32 holds S
+    [H, D, V] at its start, read at slot_read[e], written at slot_write[e].  `tail` = (source [T, C] view, taps, offset):
+    the convolution tail [taps - 1, C] at `offset` of the state is handed on from the step's rows of `source`."""
+    T = out.shape[0]
+    n_e = entry_rows.shape[0]
+    if H % qk_heads or state.dim() != 2 or state.shape[1] < H * D * V or D > 256:
+        raise KernelError("state_scan: heads, widths or state do not fit")
+    qa, ldq = _rows_view(q, "q", T, qk_heads * D)
+    ka, ldk = _rows_view(k, "k", T, qk_heads * D)
+    va, ldv = _rows_view(v, "v", T, H * V)
+    ga, ldg = _rows_view(decay, "decay", T, H * D)
+    ta, tld, tC, taps, toff = 0, 0, 0, 0, 0
+    if tail is not None:
+        src, taps, toff = tail
+        tC = src.shape[1]
+        ta, tld = _rows_view(src, "tail source", T, tC)
+        if toff < H * D * V or toff + (taps - 1) * tC > state.shape[1]:
+            raise KernelError("state_scan: the state does not hold the convolution's tail")
+    _check(lib().llmx_state_scan(qa, ldq, ka, ldk, va, ldv, ga, ldg, _dev(beta, "beta", torch.float32, (T, H)), _dev(state, "state", torch.float32),
+                                 state.shape[1], _dev(slot_read, "slot_read", torch.int32, (n_e,)), _dev(slot_write, "slot_write", torch.int32, (n_e,)),
+                                 _dev(entry_rows, "entry_rows", torch.int32, (n_e, 2)), _dev(out, "out", torch.float32, (T, H * V)), float(out_scale),
+                                 n_e, H, H // qk_heads, D, V, ta, tld, tC, int(taps), int(toff), _stream()), "state_scan")
+
+
+GATE_SIGMOID, GATE_SILU = 0, 1
+
+
+def head_norm_gate(o: torch.Tensor, weight: torch.Tensor, gate_pre: torch.Tensor, out: torch.Tensor, eps: float, H: int, V: int, gate: int) -> None:
+    """out[t, h] = o[t, h] / sqrt(mean(o[t, h]^2) + eps) * weight * gate(gate_pre[t, h]) for every head's V values; gate is
+    sigmoid or silu of a float32 view [T, H*V]; out in its own type."""
+    T = o.shape[0]
+    za, ldz = _rows_view(gate_pre, "gate_pre", T, H * V)
+    _check(lib().llmx_head_norm_gate(_dev(o, "o", torch.float32, (T, H * V)), _dev(weight, "weight", torch.float32, (V,)), za, ldz,
+                                     _dev(out, "out", shape=(T, H * V)), _code(out.dtype), float(eps), T, H, V, int(gate), _stream()), "head_norm_gate")
+
+
+def gemm_rows_view(a: torch.Tensor, w: torch.Tensor, c: torch.Tensor) -> None:
+    """c = a @ w^T for a float32 `a` whose rows may be columns of a wider tensor (a low-rank projection's inner values,
+    left in float32): the universal product with its own row stride."""
+    M, K = a.shape
+    N = w.shape[0]
+    if w.shape[1] != K or tuple(c.shape) != (M, N) or a.stride(1) != 1 or not a.is_cuda:
+        raise KernelError("gemm_rows_view: shapes do not agree")
+    lda = a.stride(0) if M > 1 else max(K, a.stride(0))
+    _check(lib().llmx_gemm_generic(a.data_ptr(), _code(a.dtype), _dev(w, "w"), _code(w.dtype), _dev(c, "c"), _code(c.dtype),
+                                   M, N, K, lda, K, N, EPI_STORE, 0, 0, 0, 1, 0, 0, 0, 0, _stream()), "gemm")
+
+
 SKINNY_MAX_ROWS = 64          # dense products of at most this many rows stream the weights once on the matrix cores
 TILE_RUNS_APART_MIN_ROWS = 17  # dense products from this many rows on take the tiled kernel with K's runs in workgroups of their own, where it offers that
 SKINNY_WIDE_MAX_ROWS = 4      # ... and of at most this many rows however wide they are
@@ -652,6 +795,36 @@ def qknorm_rope_kvwrite(qkv: torch.Tensor, q_weight: Optional[torch.Tensor], k_w
         1 if write_kv else 0, int(pairing), _stream()), "qknorm_rope_kvwrite")
 
 
+def head_norm_rope_kvwrite(qkv: torch.Tensor, bias: Optional[torch.Tensor], q_weight: Optional[torch.Tensor], k_weight: Optional[torch.Tensor],
+                           cos_sin: torch.Tensor, pos: torch.Tensor, row_entry: torch.Tensor, tables: torch.Tensor, q_out: torch.Tensor,
+                           k_cache: torch.Tensor, v_cache: torch.Tensor, eps: float, n_heads: int, n_kv_heads: int, head_dim: int,
+                           rotary_dim: int, norm_mode: int, write_kv: bool = True, pairing: int = ROPE_HALVES) -> None:
+    """qknorm_rope_kvwrite for heads that are treated one by one: float32 rows qkv = q (H*D) | k (G*D) | v (G*VD) get the
+    projections' biases (`bias`, one vector of the row's width, or None), every q and k head an RMS norm over its own dims
+    with a weight [D] shared by the heads (norm_mode QKNORM_HEAD; QKNORM_NONE: none), then the rotation; k and v go to the
+    row's page.  The value width VD is the value cache's and may differ from D."""
+    rows = qkv.shape[0]
+    n_pages, hk, page_tokens, d = k_cache.shape
+    v_dim = v_cache.shape[2]
+    width = n_heads * head_dim + n_kv_heads * head_dim + n_kv_heads * v_dim
+    if ((hk, d) != (n_kv_heads, head_dim) or tuple(v_cache.shape) != (n_pages, hk, v_dim, page_tokens) or k_cache.dtype != q_out.dtype
+            or v_cache.dtype != q_out.dtype):
+        raise KernelError("head_norm_rope_kvwrite: cache shape or dtype does not fit the heads")
+    if rotary_dim % 2 or rotary_dim > head_dim or cos_sin.shape[1] != rotary_dim:
+        raise KernelError("head_norm_rope_kvwrite: rotary width does not fit")
+    if norm_mode not in (QKNORM_NONE, QKNORM_HEAD):
+        raise KernelError("head_norm_rope_kvwrite: a norm a head, or none")
+    if norm_mode == QKNORM_HEAD:
+        _dev(q_weight, "q_weight", torch.float32, (head_dim,))
+        _dev(k_weight, "k_weight", torch.float32, (head_dim,))
+    _check(lib().llmx_head_norm_rope_kvwrite(
+        _dev(qkv, "qkv", torch.float32, (rows, width)), _dev(bias, "bias", torch.float32, (width,)), _dev(q_weight, "q_weight"),
+        _dev(k_weight, "k_weight"), _dev(cos_sin, "cos_sin", torch.float32), _dev(pos, "pos", torch.int32, (rows,)),
+        _dev(row_entry, "row_entry", torch.int32, (rows,)), _dev(tables, "tables", torch.int32), _dev(q_out, "q_out", shape=(rows, n_heads * head_dim)),
+        _dev(k_cache, "k_cache"), _dev(v_cache, "v_cache"), _code(q_out.dtype), float(eps), rows, n_heads, n_kv_heads, head_dim, v_dim,
+        rotary_dim, norm_mode, page_tokens, tables.shape[1], 1 if write_kv else 0, int(pairing), _stream()), "head_norm_rope_kvwrite")
+
+
 class AttentionPlan:
     """Work items of the matrix-core attention kernel for one step's rows (they hold no positions, so a plan serves
     every step with the same rows per request) and the merge list of the items that were split over the context."""
@@ -746,17 +919,20 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
                     tables: torch.Tensor, out: torch.Tensor, scale: float, n_heads: int, window: int = 0,
                     plan: Optional[AttentionPlan] = None, scratch=None) -> None:
     """Causal attention of each row over its request's pages.  With a `plan` (and bfloat16, head_dim a multiple of 16,
-    pages of a multiple of 16 tokens) the matrix-core kernel runs; `scratch(name, shape, dtype)` gives it storage for
-    the partial results of split contexts.  Otherwise the universal kernel runs."""
+    pages of a multiple of 16 tokens, values as wide as keys) the matrix-core kernel runs; `scratch(name, shape, dtype)`
+    gives it storage for the partial results of split contexts.  Otherwise the universal kernel runs; it takes values of
+    a width of their own (v_cache [pages, kv_heads, v_dim, page_tokens], out [rows, heads * v_dim])."""
     rows = q.shape[0]
     n_pages, n_kv_heads, page_tokens, head_dim = k_cache.shape
-    if q.shape[1] != n_heads * head_dim or out.shape != q.shape or q.dtype != k_cache.dtype or out.dtype != q.dtype:
+    v_dim = v_cache.shape[2]
+    if (q.shape[1] != n_heads * head_dim or tuple(out.shape) != (rows, n_heads * v_dim) or q.dtype != k_cache.dtype or out.dtype != q.dtype
+            or v_cache.dtype != q.dtype):
         raise KernelError("paged_attention: shapes or dtypes do not agree")
-    if head_dim > MAX_HEAD_DIM or n_heads % n_kv_heads:
-        raise KernelError(f"paged_attention: head_dim {head_dim} above {MAX_HEAD_DIM} or heads {n_heads} not a multiple of KV heads {n_kv_heads}")
-    common = (_dev(q, "q"), _dev(k_cache, "k_cache"), _dev(v_cache, "v_cache", shape=(n_pages, n_kv_heads, head_dim, page_tokens)),
+    if head_dim > MAX_HEAD_DIM or v_dim > MAX_HEAD_DIM or n_heads % n_kv_heads:
+        raise KernelError(f"paged_attention: head_dim {head_dim} or value width {v_dim} above {MAX_HEAD_DIM}, or heads {n_heads} not a multiple of KV heads {n_kv_heads}")
+    common = (_dev(q, "q"), _dev(k_cache, "k_cache"), _dev(v_cache, "v_cache", shape=(n_pages, n_kv_heads, v_dim, page_tokens)),
               _dev(pos, "pos", torch.int32, (rows,)), _dev(row_entry, "row_entry", torch.int32, (rows,)), _dev(tables, "tables", torch.int32))
-    if plan is not None and plan.n_items and attention_mfma_ok(q.dtype, head_dim, page_tokens):
+    if plan is not None and plan.n_items and v_dim == head_dim and attention_mfma_ok(q.dtype, head_dim, page_tokens):
         part_o = part_ml = None
         if plan.n_slots:
             if scratch is None:
@@ -772,7 +948,7 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
                "paged_attention_mfma")
         return
     _check(lib().llmx_paged_attention_generic(*common, _dev(out, "out"), _code(q.dtype), float(scale), rows, n_heads, n_kv_heads,
-                                              head_dim, page_tokens, tables.shape[1], int(window), _stream()), "paged_attention")
+                                              head_dim, page_tokens, tables.shape[1], int(window), v_dim, _stream()), "paged_attention")
 
 
 def _parts_args(z: torch.Tensor, parts: Optional[torch.Tensor]):
@@ -784,15 +960,16 @@ def _parts_args(z: torch.Tensor, parts: Optional[torch.Tensor]):
 
 
 def route_topk(z: torch.Tensor, bias: Optional[torch.Tensor], ids: torch.Tensor, weights: torch.Tensor, k: int, score: int,
-               normalize: bool, scale: float, parts: Optional[torch.Tensor] = None) -> None:
+               normalize: bool, scale: float, parts: Optional[torch.Tensor] = None, logit_bias: Optional[torch.Tensor] = None) -> None:
     """`parts` [slices, rows, experts]: the logits arrive as partial sums (gemm_f32's `parts`); they are added in slice
-    order into z first."""
+    order into z first.  `logit_bias` [experts]: added to the logits (z keeps the sum) before scores are formed."""
     rows, n_experts = z.shape
     if n_experts > MAX_EXPERTS or k > MAX_TOP_K or k > n_experts:
         raise KernelError(f"route_topk takes at most {MAX_EXPERTS} experts and {MAX_TOP_K} picks, not {n_experts} and {k}")
     _check(lib().llmx_route_topk(_dev(z, "z", torch.float32), *_parts_args(z, parts), _dev(bias, "bias", torch.float32, (n_experts,)),
                                  _dev(ids, "ids", torch.int32, (rows, k)), _dev(weights, "weights", torch.float32, (rows, k)),
-                                 rows, n_experts, k, score, 1 if normalize else 0, float(scale), _stream()), "route_topk")
+                                 rows, n_experts, k, score, 1 if normalize else 0, float(scale),
+                                 _dev(logit_bias, "logit_bias", torch.float32, (n_experts,)), _stream()), "route_topk")
 
 
 def moe_align_scratch(n_pairs: int, n_experts: int) -> int:
@@ -827,11 +1004,12 @@ def moe_align(ids: torch.Tensor, n_experts: int, counts: torch.Tensor, offsets: 
 def route_topk_align(z: torch.Tensor, bias: Optional[torch.Tensor], ids: torch.Tensor, weights: torch.Tensor, k: int, score: int,
                      normalize: bool, scale: float, counts: torch.Tensor, offsets: torch.Tensor, pairs: torch.Tensor,
                      active: torch.Tensor, n_active: torch.Tensor, parts: Optional[torch.Tensor] = None,
-                     scratch: Optional[torch.Tensor] = None, tile_stats: Optional[torch.Tensor] = None) -> None:
+                     scratch: Optional[torch.Tensor] = None, tile_stats: Optional[torch.Tensor] = None,
+                     logit_bias: Optional[torch.Tensor] = None) -> None:
     """route_topk followed by moe_align; a step of at most 16 rows (sigmoid scores, at most 256 experts and 64 picks) does
     both in one launch, with the same bits."""
     rows, n_experts = z.shape
-    if score == SCORE_SIGMOID and rows <= 16 and rows * k <= 1024 and n_experts <= 256 and k <= 64:
+    if score == SCORE_SIGMOID and rows <= 16 and rows * k <= 1024 and n_experts <= 256 and k <= 64 and logit_bias is None:
         _check(lib().llmx_route_topk_align(
             _dev(z, "z", torch.float32), *_parts_args(z, parts), _dev(bias, "bias", torch.float32, (n_experts,)),
             _dev(ids, "ids", torch.int32, (rows, k)),
@@ -840,7 +1018,7 @@ def route_topk_align(z: torch.Tensor, bias: Optional[torch.Tensor], ids: torch.T
             _dev(pairs, "pairs", torch.int32, (rows * k,)), _dev(active, "active", torch.int32, (n_experts,)),
             _dev(n_active, "n_active", torch.int32, (1,)), _stream()), "route_topk_align")
         return
-    route_topk(z, bias, ids, weights, k, score, normalize, scale, parts)
+    route_topk(z, bias, ids, weights, k, score, normalize, scale, parts, logit_bias)
     moe_align(ids, n_experts, counts, offsets, pairs, active, n_active, scratch, tile_stats)
 
 

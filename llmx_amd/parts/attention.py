@@ -1,7 +1,7 @@
 """Causal grouped-query softmax attention over the paged cache.
 
-Per row: q, k, v projections of the normed input (no biases); an optional RMSNorm over the whole q and the whole k
-projection; rotation of the first `rotary_dim` values of each head at the row's position; k and v written to the
+Per row: q, k, v projections of the normed input (biases optional); an optional RMSNorm over the whole q and the whole k
+projection, or over every q and k head by itself with one weight of head_dim values for all heads; rotation of the first `rotary_dim` values of each head at the row's position; k and v written to the
 request's pages; softmax(q.k * head_dim^-1/2) over keys 0..p (or the last `window`) of the same request, head h reading
 KV head h / (heads / kv_heads); output projection.  Formula order: /root/reference/src/backends/cpu/cpu_backend.hpp:971-1104
 (attention), :1461-1480 (rotation); the norm over the whole projection is this architecture's variant of the
@@ -16,14 +16,19 @@ import torch
 from .. import ops
 from ..limits import MAX_HEAD_DIM
 from .base import BuildContext, LayerCache, Mixer, build_part, register
-from .spec import KVNeed, PartSpec, TensorSpec
+from .spec import CacheTensor, KVNeed, PagedNeed, PartSpec, TensorSpec
 
-_NORM_MODES = {"none": ops.QKNORM_NONE, "projection": ops.QKNORM_PROJECTION}
+_NORM_MODES = {"none": ops.QKNORM_NONE, "projection": ops.QKNORM_PROJECTION, "head": ops.QKNORM_HEAD}
+
+# the names of an attention's tensors below its prefix; `names` in the parameters replaces any of them
+_NAMES = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "o": "o_proj.weight", "q_norm": "q_norm.weight",
+          "k_norm": "k_norm.weight", "q_bias": "q_proj.bias", "k_bias": "k_proj.bias", "v_bias": "v_proj.bias", "o_bias": "o_proj.bias"}
 
 
 class Attention(Mixer):
-    """params: hidden, heads, kv_heads, head_dim, qk_norm ("projection" | "none"), eps, window (None | int), position (PartSpec),
-    scale (None: head_dim^-1/2; else the factor the scores are multiplied by)."""
+    """params: hidden, heads, kv_heads, head_dim, qk_norm ("projection" | "head" | "none"), eps, window (None | int), position (PartSpec),
+    scale (None: head_dim^-1/2; else the factor the scores are multiplied by), v_dim (a value head's width, head_dim by
+    default), bias (True: q, k, v and the output projection have biases), names ({role: name below the prefix})."""
     graph_safe = True
 
     def __init__(self, params, prefix, ctx: BuildContext):
@@ -51,34 +56,70 @@ class Attention(Mixer):
         self.scale = float(p["scale"]) if p.get("scale") is not None else float(np.float32(1.0) / np.sqrt(np.float32(self.head_dim)))
         if not self.scale > 0.0:
             raise ValueError(f"attention: the softmax scale must be positive, not {self.scale}")
+        self.v_dim = int(p["v_dim"]) if p.get("v_dim") is not None else self.head_dim
+        if not 0 < self.v_dim <= MAX_HEAD_DIM:
+            raise ValueError(f"attention: v_dim {self.v_dim} is outside what the attention kernels take (1 to {MAX_HEAD_DIM})")
+        self.bias = bool(p.get("bias", False))
+        self.names = dict(_NAMES)
+        unknown = set(p.get("names") or {}) - set(_NAMES)
+        if unknown:
+            raise ValueError(f"attention: no tensor role named {sorted(unknown)}")
+        self.names.update(p.get("names") or {})
         self.q_width = self.heads * self.head_dim
         self.kv_width = self.kv_heads * self.head_dim
-        self.wqkv = self.wo = self.q_norm = self.k_norm = None
+        self.v_width = self.kv_heads * self.v_dim
+        self.o_width = self.heads * self.v_dim
+        # the plain case (one width, no biases, no norm a head) keeps the kernel that norms whole projections
+        self.by_head = self.norm_mode == ops.QKNORM_HEAD or self.bias or self.v_dim != self.head_dim
+        if self.by_head and self.norm_mode == ops.QKNORM_PROJECTION:
+            raise ValueError("attention: a norm over the whole projection goes with values as wide as keys and no biases")
+        self.wqkv = self.wo = self.q_norm = self.k_norm = self.b_qkv = self.b_o = None
 
     def cache_need(self):
-        return KVNeed(self.kv_heads, self.head_dim, self.window)
+        if self.v_dim == self.head_dim:
+            return KVNeed(self.kv_heads, self.head_dim, self.window)
+        return PagedNeed((CacheTensor("k", (self.kv_heads, self.head_dim), None, 1), CacheTensor("v", (self.kv_heads, self.v_dim), None, 2)),
+                         self.window)
+
+    def tensor(self, role):
+        return self.name(self.names[role])
 
     def tensor_specs(self, available):
         # one product for the three projections: the file's q, k and v go straight into the rows q | k | v of one tensor
-        fused, shape = self.name("qkv_proj.weight"), (self.q_width + 2 * self.kv_width, self.hidden)
-        q, kv = self.q_width, self.kv_width
+        q, kv, vw = self.q_width, self.kv_width, self.v_width
+        fused, shape = self.name("qkv_proj.weight"), (q + kv + vw, self.hidden)
         specs = [
-            TensorSpec(self.name("q_proj.weight"), (q, self.hidden), into=(fused, shape, (slice(0, q),))),
-            TensorSpec(self.name("k_proj.weight"), (kv, self.hidden), into=(fused, shape, (slice(q, q + kv),))),
-            TensorSpec(self.name("v_proj.weight"), (kv, self.hidden), into=(fused, shape, (slice(q + kv, q + 2 * kv),))),
-            TensorSpec(self.name("o_proj.weight"), (self.hidden, self.q_width)),
+            TensorSpec(self.tensor("q"), (q, self.hidden), into=(fused, shape, (slice(0, q),))),
+            TensorSpec(self.tensor("k"), (kv, self.hidden), into=(fused, shape, (slice(q, q + kv),))),
+            TensorSpec(self.tensor("v"), (vw, self.hidden), into=(fused, shape, (slice(q + kv, q + kv + vw),))),
+            TensorSpec(self.tensor("o"), (self.hidden, self.o_width)),
         ]
         if self.norm_mode == ops.QKNORM_PROJECTION:
-            specs += [TensorSpec(self.name("q_norm.weight"), (self.q_width,), "norm"),
-                      TensorSpec(self.name("k_norm.weight"), (self.kv_width,), "norm")]
+            specs += [TensorSpec(self.tensor("q_norm"), (q,), "norm"), TensorSpec(self.tensor("k_norm"), (kv,), "norm")]
+        elif self.norm_mode == ops.QKNORM_HEAD:
+            specs += [TensorSpec(self.tensor("q_norm"), (self.head_dim,), "norm"), TensorSpec(self.tensor("k_norm"), (self.head_dim,), "norm")]
+        if self.bias:
+            fused_b, shape_b = self.name("qkv_proj.bias"), (q + kv + vw,)
+            specs += [TensorSpec(self.tensor("q_bias"), (q,), "bias", into=(fused_b, shape_b, (slice(0, q),))),
+                      TensorSpec(self.tensor("k_bias"), (kv,), "bias", into=(fused_b, shape_b, (slice(q, q + kv),))),
+                      TensorSpec(self.tensor("v_bias"), (vw,), "bias", into=(fused_b, shape_b, (slice(q + kv, q + kv + vw),))),
+                      TensorSpec(self.tensor("o_bias"), (self.hidden,), "bias")]
         return specs
 
     def load(self, tensors):
         self.wqkv = tensors[self.name("qkv_proj.weight")]
-        self.wo = tensors[self.name("o_proj.weight")]
-        if self.norm_mode == ops.QKNORM_PROJECTION:
-            self.q_norm = tensors[self.name("q_norm.weight")]
-            self.k_norm = tensors[self.name("k_norm.weight")]
+        self.wo = tensors[self.tensor("o")]
+        if self.norm_mode != ops.QKNORM_NONE:
+            self.q_norm = tensors[self.tensor("q_norm")]
+            self.k_norm = tensors[self.tensor("k_norm")]
+        if self.bias:
+            self.b_qkv = tensors[self.name("qkv_proj.bias")]
+            self.b_o = tensors[self.tensor("o_bias")]
+
+    def output_bias(self):
+        """The output projection's bias, which a caller that joins this mixer's result with others may add itself
+        (forward(..., add_output_bias=False)); None without one."""
+        return self.b_o
 
     def takes_deferred_norm(self, step):
         return ops.gemm_takes_normed_rows(step.rows, self.wqkv, torch.float32)
@@ -94,24 +135,37 @@ class Attention(Mixer):
     def graph_key(self, step):
         # a recorded step holds the plan's addresses and launch sizes; the universal kernel has no plan
         page = self.ctx.page_tokens
-        return self._plan(step) if page and ops.attention_mfma_ok(step.act_dtype, self.head_dim, page) else None
+        return self._plan(step) if page and self._mfma(step.act_dtype, page) else None
 
-    def forward(self, step, h, out, accumulate, cache: LayerCache, h32=None):
+    def _mfma(self, act, page_tokens):
+        return self.v_dim == self.head_dim and ops.attention_mfma_ok(act, self.head_dim, page_tokens)
+
+    def forward(self, step, h, out, accumulate, cache: LayerCache, h32=None, add_output_bias=True):
         T = step.rows
         act = step.act_dtype
-        qkv = step.buf("attention.qkv", (T, self.q_width + 2 * self.kv_width), torch.float32)
+        qkv = step.buf("attention.qkv", (T, self.q_width + self.kv_width + self.v_width), torch.float32)
         ops.gemm(h, self.wqkv, qkv, scratch=step.buf)
         q = step.buf("attention.q", (T, self.q_width), act)
         cos_sin, rotary = self.position.rotation()
         tables = step.tables(cache.group)
-        ops.qknorm_rope_kvwrite(qkv, self.q_norm, self.k_norm, cos_sin, step.positions, step.row_entry, tables, q, cache.k, cache.v,
-                                self.eps, self.heads, self.kv_heads, self.head_dim, rotary, self.norm_mode, write_kv=cache.writes,
-                                pairing=self.pairing)
-        o = step.buf("attention.out", (T, self.q_width), act)
-        plan = self._plan(step) if ops.attention_mfma_ok(act, self.head_dim, cache.k.shape[2]) else None
+        if self.by_head:
+            ops.head_norm_rope_kvwrite(qkv, self.b_qkv, self.q_norm, self.k_norm, cos_sin, step.positions, step.row_entry, tables, q, cache.k,
+                                       cache.v, self.eps, self.heads, self.kv_heads, self.head_dim, rotary, self.norm_mode,
+                                       write_kv=cache.writes, pairing=self.pairing)
+        else:
+            ops.qknorm_rope_kvwrite(qkv, self.q_norm, self.k_norm, cos_sin, step.positions, step.row_entry, tables, q, cache.k, cache.v,
+                                    self.eps, self.heads, self.kv_heads, self.head_dim, rotary, self.norm_mode, write_kv=cache.writes,
+                                    pairing=self.pairing)
+        o = step.buf("attention.out", (T, self.o_width), act)
+        plan = self._plan(step) if self._mfma(act, cache.k.shape[2]) else None
         ops.paged_attention(q, cache.k, cache.v, step.positions, step.row_entry, tables, o, self.scale, self.heads,
                             window=int(self.window or 0), plan=plan, scratch=step.buf)
-        ops.gemm(o, self.wo, out, ops.EPI_ADD if accumulate else ops.EPI_STORE, scratch=step.buf)
+        if self.b_o is not None and add_output_bias:
+            y = step.buf("attention.projected", (T, self.hidden), torch.float32)
+            ops.gemm(o, self.wo, y, scratch=step.buf)
+            ops.combine_rows(out, y, 1.0, self.b_o, accumulate=accumulate)
+        else:
+            ops.gemm(o, self.wo, out, ops.EPI_ADD if accumulate else ops.EPI_STORE, scratch=step.buf)
 
 
 register("mixer", "attention", Attention)

@@ -29,7 +29,7 @@ from typing import Callable, Dict, List, Optional, Sequence, Set, Union
 
 import torch
 
-from .spec import PagedNeed, PartSpec, StateNeed, TensorSpec
+from .spec import CompositeNeed, PagedNeed, PartSpec, StateNeed, TensorSpec
 
 
 @dataclass
@@ -109,6 +109,7 @@ class LayerCache:
     tensors: Optional[Dict[str, torch.Tensor]] = None   # name -> [pages, *CacheTensor.page_shape(page_tokens)]
     writes: bool = True                      # False: this entry reads pages another entry wrote
     state: Optional[torch.Tensor] = None     # [slots, *StateNeed.shape]
+    members: Optional[list] = None           # a composite need's members' caches (LayerCache or None each), in their order
 
     @property
     def k(self) -> torch.Tensor:
@@ -132,7 +133,7 @@ class Mixer(Part):
         """Whether, for this step, forward accepts a Norm.deferred() description as h and h32 in place of tensors."""
         return False
 
-    def cache_need(self) -> Union[PagedNeed, StateNeed, None]:
+    def cache_need(self) -> Union[PagedNeed, StateNeed, CompositeNeed, None]:
         return None
 
     def forward(self, step, h: torch.Tensor, out: torch.Tensor, accumulate: bool, cache: LayerCache,

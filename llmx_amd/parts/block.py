@@ -4,6 +4,8 @@
 /root/reference/src/model/arch/minimax_m3.hpp:247-287 (norm, mixer joined into the residual, norm, feed-forward joined).
 "parallel": x += s1 * mixer(norm1(x)) + s2 * ffn(norm2(x)) with both norms of the same x, learned factors s1, s2 a
 coordinate, and an optional per-layer token input after the sum.
+"outnorm": x += norm1(mixer(x)); x += norm2(ffn(x)): the sublayers read the residual itself and only their results are
+normed.
 """
 
 from __future__ import annotations
@@ -130,6 +132,51 @@ class ParallelBlock:
             self.token_input.forward(step, x, copy)
 
 
+class OutNormBlock:
+    """x += mixer_norm(mixer(x)); x += ffn_norm(ffn(x)), the feed-forward (with its norm) optional.  The sublayers read x
+    itself: in the serving path its rounded copy, which the join before them writes on its way (`add_into(..., copy)`), so
+    that only a model's first layer needs a launch for it; the router of a routed feed-forward still gets the unrounded
+    rows.  The norms are parts of the "norm" family that have `add_into` (x += norm(y))."""
+    graph_safe = True
+
+    def __init__(self, spec: BlockSpec, ctx: BuildContext):
+        if (spec.ffn is None) != (spec.ffn_norm is None):
+            raise ValueError("outnorm block: a feed-forward comes with its norm, and a norm with its feed-forward")
+        self.mixer_norm = build_part("norm", spec.mixer_norm, ctx)
+        self.mixer = build_part("mixer", spec.mixer, ctx)
+        self.ffn_norm = build_part("norm", spec.ffn_norm, ctx) if spec.ffn_norm is not None else None
+        self.ffn = build_part("feed_forward", spec.ffn, ctx) if spec.ffn is not None else None
+        for n in (self.mixer_norm, self.ffn_norm):
+            if n is not None and not hasattr(n, "add_into"):
+                raise ValueError(f"outnorm block: the norm {n.kind!r} cannot join a result into the residual (no add_into)")
+        if spec.extra:
+            raise ValueError(f"outnorm block: no slot named {sorted(spec.extra)}")
+
+    def parts(self):
+        return [p for p in (self.mixer_norm, self.mixer, self.ffn_norm, self.ffn) if p is not None]
+
+    def forward(self, step, x: torch.Tensor, cache: LayerCache) -> None:
+        T, E = x.shape
+        exact = step.act_dtype == torch.float32
+        if exact:
+            h = x                                   # the sublayers write elsewhere, so they may read the residual in place
+        else:
+            h = step.buf("block.x_act", (T, E), step.act_dtype)
+            fresh = step.shared("outnorm.copy", dict)       # which run-order entry the copy was written for
+            if fresh.get("for") != step.run_index:
+                ops.cast_rows(x, h)
+        y = step.buf("block.y", (T, E), torch.float32)
+        self.mixer.forward(step, h, y, False, cache, x if self.mixer.wants_f32_input else None)
+        last = self.ffn is None
+        self.mixer_norm.add_into(step, x, y, None if exact else h)
+        if not last:
+            self.ffn.forward(step, h, y, False, x if self.ffn.wants_f32_input else None)
+            self.ffn_norm.add_into(step, x, y, None if exact else h)
+        if not exact:
+            step.shared("outnorm.copy", dict)["for"] = step.run_index + 1
+
+
 register("block", "prenorm", PreNormBlock)
+register("block", "outnorm", OutNormBlock)
 register("block", "parallel", ParallelBlock)
 register("scale", "layer_scale", LayerScale)

@@ -44,7 +44,8 @@ class TokenEmbedding(Embedding):
 
 
 class LinearHead(Head):
-    """params: vocab, hidden, tied (bool); tensor (the name's last part, "weight" by default).
+    """params: vocab, hidden, tied (bool); tensor (the name's last part, "weight" by default); logit_scale (the logits are
+    multiplied by it, 1 by default) and softcap (c > 0: logits <- c tanh(logits / c), after the scale; None: none).
     Tensor <prefix><tensor> (vocab, hidden) unless tied."""
     graph_safe = True
 
@@ -54,6 +55,10 @@ class LinearHead(Head):
         self.hidden = int(params["hidden"])
         self.tied = bool(params.get("tied", False))
         self.tensor = str(params.get("tensor", "weight"))
+        self.logit_scale = float(params.get("logit_scale", 1.0))
+        self.softcap = float(params["softcap"]) if params.get("softcap") else 0.0
+        if self.softcap < 0.0:
+            raise ValueError("head: a softcap is positive")
         self.weight = None
 
     def tensor_specs(self, available):
@@ -68,6 +73,8 @@ class LinearHead(Head):
 
     def forward(self, step, rows, logits):
         ops.gemm(rows, self.weight, logits)
+        if self.logit_scale != 1.0 or self.softcap > 0.0:
+            ops.scale_softcap(logits, self.logit_scale, self.softcap)
 
 
 register("embedding", "token_embedding", TokenEmbedding)

@@ -1,0 +1,154 @@
+"""Mixers that carry a float32 matrix state S [key channels D, value channels V] a head from token to token.
+
+Both decay S's rows channel by channel and add an outer product a token; they differ in what is added:
+    S_t = diag(g_t) S_(t-1) + k_t u_t^T,   o_t = S_t^T q_t
+    gated linear attention:  u_t = v_t,                               g_t = sigmoid(z_t)^(1/tau)
+    gated delta rule:        u_t = beta_t (v_t - (diag(g_t) S_(t-1))^T k_t),   g_t = exp(-exp(A) softplus(step_t + dt_bias))
+with z_t and step_t low-rank projections of the input.  The delta rule's q, k and v first pass a short causal convolution
+over time and silu, and q and k are made unit vectors a head.  The read-out is RMS-normed a head, gated, and projected.
+Products may read rounded rows; decays, gates, unit norms, the recurrence and the state are float32 in both paths.
+The state lives in the request's slot: S [H, D, V], then (delta rule) the convolution's last taps - 1 inputs [taps - 1, C].
+"""
+
+from __future__ import annotations
+
+import torch
+
+from .. import ops
+from .base import LayerCache, Mixer, register
+from .spec import StateNeed, TensorSpec
+
+
+class GatedLinearAttention(Mixer):
+    """params: hidden, heads, dim, vdim, tau, eps, rank (the decay projection's inner width).
+    q = W_q h * dim^-1/2, k = W_k h, v = W_v h; decay = sigmoid(W_a2 (W_a1 h) + b)^(1/tau) a key channel;
+    result = W_o (rmsnorm_head(o) * w * silu(W_g h)).  Tensors <prefix>q, k, v, g, o, norm, a1, a2, a2.b."""
+    graph_safe = True
+    steps_between_slots = True      # reads the state at step.entry_held_slots, writes it at step.entry_slots
+
+    def __init__(self, params, prefix, ctx):
+        super().__init__(params, prefix, ctx)
+        p = params
+        self.hidden, self.heads, self.dim, self.vdim = int(p["hidden"]), int(p["heads"]), int(p["dim"]), int(p["vdim"])
+        self.rank = int(p["rank"])
+        self.tau, self.eps = float(p["tau"]), float(p["eps"])
+        if min(self.heads, self.dim, self.vdim, self.rank) < 1 or self.dim > 256 or not self.tau > 0.0:
+            raise ValueError("gated linear attention: heads, dim (at most 256), vdim and rank are at least 1 and tau is positive")
+        HD, HV = self.heads * self.dim, self.heads * self.vdim
+        # the fused in-projection's columns: q | k | v | g | a1
+        self.cols = {"q": (0, HD), "k": (HD, HD), "v": (2 * HD, HV), "g": (2 * HD + HV, HV), "a1": (2 * HD + 2 * HV, self.rank)}
+        self.in_width = 2 * HD + 2 * HV + self.rank
+        self.w_in = self.w_a2 = self.b_a2 = self.w_o = self.norm = None
+
+    def cache_need(self):
+        return StateNeed((self.heads * self.dim * self.vdim,), "float32")
+
+    def tensor_specs(self, available):
+        E = self.hidden
+        fused, shape = self.name("in"), (self.in_width, E)
+        specs = [TensorSpec(self.name(n), (w, E), into=(fused, shape, (slice(at, at + w),))) for n, (at, w) in self.cols.items()]
+        return specs + [TensorSpec(self.name("a2"), (self.heads * self.dim, self.rank)),
+                        TensorSpec(self.name("a2.b"), (self.heads * self.dim,), "bias"),
+                        TensorSpec(self.name("norm"), (self.vdim,), "norm"),
+                        TensorSpec(self.name("o"), (E, self.heads * self.vdim))]
+
+    def load(self, tensors):
+        self.w_in = tensors[self.name("in")]
+        self.w_a2, self.b_a2 = tensors[self.name("a2")], tensors[self.name("a2.b")]
+        self.norm, self.w_o = tensors[self.name("norm")], tensors[self.name("o")]
+
+    def forward(self, step, h, out, accumulate, cache: LayerCache, h32=None):
+        T, H, D, V = step.rows, self.heads, self.dim, self.vdim
+        pre = step.buf("gla.pre", (T, self.in_width), torch.float32)
+        ops.gemm(h, self.w_in, pre, scratch=step.buf)
+        view = lambda n: pre[:, self.cols[n][0]:self.cols[n][0] + self.cols[n][1]]
+        z = step.buf("gla.z", (T, H * D), torch.float32)
+        ops.gemm_rows_view(view("a1"), self.w_a2, z)
+        decay = step.buf("gla.decay", (T, H * D), torch.float32)
+        ops.sigmoid_root(z, self.b_a2, self.tau, decay)
+        o = step.buf("gla.o", (T, H * V), torch.float32)
+        ops.state_scan(view("q"), view("k"), view("v"), decay, None, cache.state, step.entry_held_slots, step.entry_slots, step.entry_rows, o,
+                       float(D) ** -0.5, H, H, D, V)
+        gated = step.buf("gla.gated", (T, H * V), step.act_dtype)
+        ops.head_norm_gate(o, self.norm, view("g"), gated, self.eps, H, V, ops.GATE_SILU)
+        ops.gemm(gated, self.w_o, out, ops.EPI_ADD if accumulate else ops.EPI_STORE, scratch=step.buf)
+
+
+class ChannelDeltaRule(Mixer):
+    """params: hidden, heads, kv_heads (q and k heads; head h reads q/k head h / (heads / kv_heads)), dim, vdim, conv (taps),
+    eps, decay_rank, gate_rank.  Tensors <prefix>q, k, v (+ .conv [channels, taps]), b, A_log, dt_bias, a1, a2, g1, g2,
+    norm, o.  result = W_o (rmsnorm_head(o) * w * sigmoid(W_g2 (W_g1 h)))."""
+    graph_safe = True
+    steps_between_slots = True
+
+    def __init__(self, params, prefix, ctx):
+        super().__init__(params, prefix, ctx)
+        p = params
+        self.hidden, self.heads, self.kv_heads = int(p["hidden"]), int(p["heads"]), int(p["kv_heads"])
+        self.dim, self.vdim, self.taps = int(p["dim"]), int(p["vdim"]), int(p["conv"])
+        self.decay_rank, self.gate_rank = int(p["decay_rank"]), int(p["gate_rank"])
+        self.eps = float(p["eps"])
+        if min(self.heads, self.kv_heads, self.dim, self.vdim, self.taps, self.decay_rank, self.gate_rank) < 1 or self.dim > 256:
+            raise ValueError("delta rule: heads, kv_heads, dim (at most 256), vdim, conv and the ranks are at least 1")
+        if self.heads % self.kv_heads:
+            raise ValueError("delta rule: the head count must be divisible by the q/k head count")
+        GD, HV, H = self.kv_heads * self.dim, self.heads * self.vdim, self.heads
+        self.channels = 2 * GD + HV
+        if self.channels * 4 > 64 * 1024:
+            raise ValueError(f"delta rule: {self.channels} convolved channels a row; the preparation kernel keeps at most {64 * 1024 // 4}")
+        # the fused in-projection's columns: q | k | v (the convolved channels, in this order) | b | a1 | g1
+        self.cols = {"q": (0, GD), "k": (GD, GD), "v": (2 * GD, HV), "b": (self.channels, H), "a1": (self.channels + H, self.decay_rank),
+                     "g1": (self.channels + H + self.decay_rank, self.gate_rank)}
+        self.in_width = self.channels + H + self.decay_rank + self.gate_rank
+        self.state_matrix = H * self.dim * self.vdim
+        self.w_in = self.conv = self.a_log = self.dt_bias = self.w_a2 = self.w_g2 = self.norm = self.w_o = None
+
+    def cache_need(self):
+        return StateNeed((self.state_matrix + (self.taps - 1) * self.channels,), "float32")
+
+    def tensor_specs(self, available):
+        E, H, D, V = self.hidden, self.heads, self.dim, self.vdim
+        fused, shape = self.name("in"), (self.in_width, E)
+        specs = [TensorSpec(self.name(n), (w, E), into=(fused, shape, (slice(at, at + w),))) for n, (at, w) in self.cols.items()]
+        taps_of, taps_shape = self.name("conv"), (self.channels, self.taps)
+        specs += [TensorSpec(self.name(f"{n}.conv"), (self.cols[n][1], self.taps), "bias",
+                             into=(taps_of, taps_shape, (slice(self.cols[n][0], self.cols[n][0] + self.cols[n][1]),)), init=("uniform", -0.5, 0.5))
+                  for n in ("q", "k", "v")]
+        return specs + [TensorSpec(self.name("A_log"), (H,), "bias", init=("uniform", -1.0, 1.0)),
+                        TensorSpec(self.name("dt_bias"), (H * D,), "bias"),
+                        TensorSpec(self.name("a2"), (H * D, self.decay_rank)),
+                        TensorSpec(self.name("g2"), (H * V, self.gate_rank)),
+                        TensorSpec(self.name("norm"), (V,), "norm"),
+                        TensorSpec(self.name("o"), (E, H * V))]
+
+    def load(self, tensors):
+        self.w_in, self.conv = tensors[self.name("in")], tensors[self.name("conv")]
+        self.a_log, self.dt_bias = tensors[self.name("A_log")], tensors[self.name("dt_bias")]
+        self.w_a2, self.w_g2 = tensors[self.name("a2")], tensors[self.name("g2")]
+        self.norm, self.w_o = tensors[self.name("norm")], tensors[self.name("o")]
+
+    def forward(self, step, h, out, accumulate, cache: LayerCache, h32=None):
+        T, H, G, D, V = step.rows, self.heads, self.kv_heads, self.dim, self.vdim
+        f32 = torch.float32
+        pre = step.buf("delta.pre", (T, self.in_width), f32)
+        ops.gemm(h, self.w_in, pre, scratch=step.buf)
+        view = lambda n: pre[:, self.cols[n][0]:self.cols[n][0] + self.cols[n][1]]
+        step_pre = step.buf("delta.step", (T, H * D), f32)
+        ops.gemm_rows_view(view("a1"), self.w_a2, step_pre)
+        gate_pre = step.buf("delta.gate", (T, H * V), f32)
+        ops.gemm_rows_view(view("g1"), self.w_g2, gate_pre)
+        q, k = step.buf("delta.q", (T, G * D), f32), step.buf("delta.k", (T, G * D), f32)
+        v, decay, beta = step.buf("delta.v", (T, H * V), f32), step.buf("delta.decay", (T, H * D), f32), step.buf("delta.beta", (T, H), f32)
+        ops.delta_prep(pre, self.conv, step_pre, self.dt_bias, self.a_log, cache.state, self.state_matrix, step.entry_held_slots,
+                       step.row_entry, step.entry_rows, q, k, v, decay, beta, G, H, D, V, self.cols["b"][0])
+        o = step.buf("delta.o", (T, H * V), f32)
+        tail = (pre[:, :self.channels], self.taps, self.state_matrix) if self.taps > 1 else None
+        ops.state_scan(q, k, v, decay, beta, cache.state, step.entry_held_slots, step.entry_slots, step.entry_rows, o, float(D) ** -0.5,
+                       H, G, D, V, tail=tail)
+        gated = step.buf("delta.gated", (T, H * V), step.act_dtype)
+        ops.head_norm_gate(o, self.norm, gate_pre, gated, self.eps, H, V, ops.GATE_SIGMOID)
+        ops.gemm(gated, self.w_o, out, ops.EPI_ADD if accumulate else ops.EPI_STORE, scratch=step.buf)
+
+
+register("mixer", "gated_linear_attention", GatedLinearAttention)
+register("mixer", "channel_delta_rule", ChannelDeltaRule)

@@ -21,9 +21,28 @@ from .spec import TensorSpec
 
 _SCORES = {"sigmoid": ops.SCORE_SIGMOID, "softmax": ops.SCORE_SOFTMAX}
 
+# the names of a routed feed-forward's tensors below its prefix ({e}: the expert's number); `names` in the parameters
+# replaces any of them
+_EXPERT_NAMES = {"router": "gate.weight", "correction_bias": "gate.e_score_correction_bias", "logit_bias": "gate.bias",
+                 "fused_gate_up": "experts.gate_up_proj", "fused_down": "experts.down_proj",
+                 "expert_gate": "experts.{e}.gate_proj.weight", "expert_up": "experts.{e}.up_proj.weight",
+                 "expert_down": "experts.{e}.down_proj.weight"}
+_GLU_NAMES = {"gate": "gate_proj.weight", "up": "up_proj.weight", "down": "down_proj.weight"}
+
+
+def _names(defaults: dict, given, what: str) -> dict:
+    unknown = set(given or {}) - set(defaults)
+    if unknown:
+        raise ValueError(f"{what}: no tensor role named {sorted(unknown)}")
+    out = dict(defaults)
+    out.update(given or {})
+    return out
+
 
 class RoutedExperts(FeedForward):
-    """params: hidden, experts, top_k, intermediate, score ("sigmoid" | "softmax"), correction_bias (bool), normalize (bool), scale."""
+    """params: hidden, experts, top_k, intermediate, score ("sigmoid" | "softmax"), correction_bias (bool: a bias on the pick
+    keys only), logit_bias (bool: a bias that is part of the router's logits), normalize (bool), scale, names ({role: name
+    below the prefix}).  score "softmax" with normalize is the softmax over the picked logits alone."""
     graph_safe = True
 
     wants_f32_input = True
@@ -39,6 +58,8 @@ class RoutedExperts(FeedForward):
             raise ValueError(f"router score {p.get('score')!r} is not one of {sorted(_SCORES)}")
         self.score = _SCORES[p.get("score", "sigmoid")]
         self.use_bias = bool(p.get("correction_bias", False))
+        self.use_logit_bias = bool(p.get("logit_bias", False))
+        self.names = _names(_EXPERT_NAMES, p.get("names"), "routed experts")
         self.normalize = bool(p.get("normalize", True))
         self.scale = float(p.get("scale", 1.0))
         if not 0 < self.top_k <= self.experts:
@@ -47,37 +68,43 @@ class RoutedExperts(FeedForward):
             raise ValueError(f"routed experts: {self.experts} experts with {self.top_k} picks a token; the routing kernels take at most "
                              f"{MAX_EXPERTS} experts and {MAX_TOP_K} picks")
         self.per_expert = False
-        self.w_router = self.bias = self.w_gate_up = self.w_down = None
+        self.w_router = self.bias = self.logit_bias = self.w_gate_up = self.w_down = None
 
     def tensor_specs(self, available):
         X, F, E = self.experts, self.intermediate, self.hidden
-        specs = [TensorSpec(self.name("gate.weight"), (X, E), "router")]
+        nm = lambda role, **kw: self.name(self.names[role].format(**kw))
+        specs = [TensorSpec(nm("router"), (X, E), "router")]
         if self.use_bias:
-            specs.append(TensorSpec(self.name("gate.e_score_correction_bias"), (X,), "bias"))
-        fused = self.name("experts.gate_up_proj")
-        single = re.compile(re.escape(self.name("experts.")) + r"\d+\.")
+            specs.append(TensorSpec(nm("correction_bias"), (X,), "bias"))
+        if self.use_logit_bias:
+            specs.append(TensorSpec(nm("logit_bias"), (X,), "bias"))
+        fused = nm("fused_gate_up")
+        head, _, tail = self.names["expert_gate"].partition("{e}")
+        single = re.compile(re.escape(self.name(head)) + r"\d+" + re.escape(tail) + "$")
         has_single = any(single.match(n) for n in available)
         if has_single and fused in available:
             raise ValueError(f"{self.prefix}experts holds both fused and per-expert tensors")
         self.per_expert = has_single
         if has_single:
             # each expert's tensors go from the host straight into their places in the fused tensors
-            down = self.name("experts.down_proj")
+            down = nm("fused_down")
             for e in range(X):
-                specs += [TensorSpec(self.name(f"experts.{e}.gate_proj.weight"), (F, E), into=(fused, (X, 2 * F, E), (e, slice(0, F)))),
-                          TensorSpec(self.name(f"experts.{e}.up_proj.weight"), (F, E), into=(fused, (X, 2 * F, E), (e, slice(F, 2 * F)))),
-                          TensorSpec(self.name(f"experts.{e}.down_proj.weight"), (E, F), into=(down, (X, E, F), (e,)))]
+                specs += [TensorSpec(nm("expert_gate", e=e), (F, E), into=(fused, (X, 2 * F, E), (e, slice(0, F)))),
+                          TensorSpec(nm("expert_up", e=e), (F, E), into=(fused, (X, 2 * F, E), (e, slice(F, 2 * F)))),
+                          TensorSpec(nm("expert_down", e=e), (E, F), into=(down, (X, E, F), (e,)))]
         else:
-            specs += [TensorSpec(fused, (X, 2 * F, E)), TensorSpec(self.name("experts.down_proj"), (X, E, F))]
+            specs += [TensorSpec(fused, (X, 2 * F, E)), TensorSpec(nm("fused_down"), (X, E, F))]
         return specs
 
     def load(self, tensors):
-        self.w_router = tensors[self.name("gate.weight")]
+        self.w_router = tensors[self.name(self.names["router"])]
         if self.use_bias:
-            self.bias = tensors[self.name("gate.e_score_correction_bias")]
+            self.bias = tensors[self.name(self.names["correction_bias"])]
+        if self.use_logit_bias:
+            self.logit_bias = tensors[self.name(self.names["logit_bias"])]
         # per-expert files arrive fused too (see tensor_specs)
-        self.w_gate_up = tensors[self.name("experts.gate_up_proj")]
-        self.w_down = tensors[self.name("experts.down_proj")]
+        self.w_gate_up = tensors[self.name(self.names["fused_gate_up"])]
+        self.w_down = tensors[self.name(self.names["fused_down"])]
 
     def takes_deferred_norm(self, step):
         return (ops.gemm_takes_normed_rows(step.rows, self.w_gate_up, step.act_dtype, ops.EPI_SWIGLU, grouped=True)
@@ -101,7 +128,7 @@ class RoutedExperts(FeedForward):
         # for steps of many pairs the grouping also counts the experts' tiles of 128 rows, by which the products choose their tiles
         tile_stats = step.buf("experts.tile_stats", (1,), torch.int32) if T * k >= ops.TILE_STATS_MIN_PAIRS else None
         ops.route_topk_align(z, self.bias, ids, weights, k, self.score, self.normalize, self.scale, counts, offsets, pairs, active, n_active,
-                             parts=parts, scratch=scratch, tile_stats=tile_stats)
+                             parts=parts, scratch=scratch, tile_stats=tile_stats, logit_bias=self.logit_bias)
         step.observe("routing", logits=z, ids=ids, weights=weights)
         act = step.buf("experts.act", (T * k, self.intermediate), step.act_dtype)
         ops.grouped_gemm(h, self.w_gate_up, act, offsets, pairs, k, ops.EPI_SWIGLU, active, n_active, token_rows=T, tile_stats=tile_stats)
@@ -111,25 +138,27 @@ class RoutedExperts(FeedForward):
 
 
 class DenseGLU(FeedForward):
-    """params: hidden, intermediate.  y = (silu(h.Wg^T) * (h.Wu^T)).Wd^T; tensors gate_proj, up_proj, down_proj (.weight)."""
+    """params: hidden, intermediate, names ({role: name below the prefix}).  y = (silu(h.Wg^T) * (h.Wu^T)).Wd^T; tensors
+    gate_proj, up_proj, down_proj (.weight) unless named otherwise."""
     graph_safe = True
 
     def __init__(self, params, prefix, ctx):
         super().__init__(params, prefix, ctx)
         self.hidden = int(params["hidden"])
         self.intermediate = int(params["intermediate"])
+        self.names = _names(_GLU_NAMES, params.get("names"), "dense GLU")
         self.w_gate_up = self.w_down = None
 
     def tensor_specs(self, available):
         F, E = self.intermediate, self.hidden
         fused = self.name("gate_up_proj.weight")     # gate rows, then up rows, filled from the file's two tensors
-        return [TensorSpec(self.name("gate_proj.weight"), (F, E), into=(fused, (2 * F, E), (slice(0, F),))),
-                TensorSpec(self.name("up_proj.weight"), (F, E), into=(fused, (2 * F, E), (slice(F, 2 * F),))),
-                TensorSpec(self.name("down_proj.weight"), (E, F))]
+        return [TensorSpec(self.name(self.names["gate"]), (F, E), into=(fused, (2 * F, E), (slice(0, F),))),
+                TensorSpec(self.name(self.names["up"]), (F, E), into=(fused, (2 * F, E), (slice(F, 2 * F),))),
+                TensorSpec(self.name(self.names["down"]), (E, F))]
 
     def load(self, tensors):
         self.w_gate_up = tensors[self.name("gate_up_proj.weight")]
-        self.w_down = tensors[self.name("down_proj.weight")]
+        self.w_down = tensors[self.name(self.names["down"])]
 
     def takes_deferred_norm(self, step):
         return ops.gemm_takes_normed_rows(step.rows, self.w_gate_up, step.act_dtype, ops.EPI_SWIGLU)

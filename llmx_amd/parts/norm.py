@@ -1,4 +1,5 @@
-"""RMSNorm: y = x * (r * w), r = 1/sqrt(mean(x^2) + eps), all in float32.
+"""Norms of float32 rows.  RMSNorm: y = x * (r * w), r = 1/sqrt(mean(x^2) + eps); LayerNorm (a weight, no bias):
+y = (x - mean) / sqrt(var + eps) * w, var the mean of the squared deviations.  All in float32.
 
 Order of operations as the reference computes it (/root/reference/src/backends/cpu/cpu_backend.hpp:1437-1459): the
 reciprocal root times the weight is formed first, then multiplied into x.
@@ -52,4 +53,32 @@ class RMSNorm(Norm):
         return ops.NormedRows(x, self.weight, self.eps)
 
 
+class LayerNorm(Norm):
+    """params: width, eps; tensor (the name's last part, "weight" by default; "" when the prefix is the whole name).
+    Tensor: <prefix><tensor>, (width,).  `add_into` is the form an arrangement uses that norms a sublayer's result on its
+    way into the residual."""
+    graph_safe = True
+
+    def __init__(self, params, prefix, ctx):
+        super().__init__(params, prefix, ctx)
+        self.width = int(params["width"])
+        self.eps = float(params["eps"])
+        self.tensor = str(params.get("tensor", "weight"))
+        self.weight: Optional[torch.Tensor] = None
+
+    def tensor_specs(self, available):
+        return [TensorSpec(self.name(self.tensor), (self.width,), "norm")]
+
+    def load(self, tensors):
+        self.weight = tensors[self.name(self.tensor)]
+
+    def forward(self, step, x, out, out32=None, pick=None):
+        ops.layernorm(x, self.weight, self.eps, out, out32, pick)
+
+    def add_into(self, step, x, y, copy=None):
+        """x += norm(y); `copy` (optional) receives the new rows in its own type."""
+        ops.layernorm_add(x, y, self.weight, self.eps, copy)
+
+
 register("norm", "rmsnorm", RMSNorm)
+register("norm", "layernorm", LayerNorm)

@@ -135,6 +135,22 @@ class StateNeed:
     dtype: str = "float32"
 
 
+@dataclass(frozen=True)
+class CompositeNeed:
+    """A mixer made of several mixers that run side by side, each with a need of its own (pages for one, a state for
+    another): the needs in the members' order, None for a member that keeps nothing.  The engine gives every member what a
+    mixer alone would get (a paged member joins the cache group of its need, a state member gets slots) and hands the
+    mixer a `LayerCache` whose `members` are theirs."""
+    members: Tuple[Any, ...]
+
+    def leaves(self):
+        for m in self.members:
+            if isinstance(m, CompositeNeed):
+                yield from m.leaves()
+            else:
+                yield m
+
+
 @dataclass
 class ModelSpec:
     architecture: str
