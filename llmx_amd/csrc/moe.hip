@@ -96,7 +96,8 @@ __device__ __forceinline__ void route_row_256(const float (&x)[4], const float (
 
 // One wave per row.  score s_e = sigmoid(z_e) (or softmax over the row); the pick key is b_e = s_e + bias_e; k times
 // the largest key not yet taken is picked, the lowest id on ties; the weight is the unbiased s_e, divided by the
-// picks' sum (added in pick order) when `normalize`, then times `scale`.  A row with a non-finite key gets ids -1 and
+// picks' sum (added in pick order) when `normalize` (1: a single softmax pick keeps its score; 2: it too is divided, so its
+// weight is 1: the softmax over the picked logits alone), then times `scale`.  A row with a non-finite key gets ids -1 and
 // weights 0.  Ids and weights come out in pick order, best first.
 // `logit_bias` (optional): added to the logits (and kept in z) before anything else: a router whose bias is part of its
 // logits, so that scores and weights see it too.
@@ -186,7 +187,7 @@ __global__ void __launch_bounds__(64) route_topk_kernel(float* __restrict__ z, c
     if (lane == 0) {
         float total = 0.0f;
         for (int j = 0; j < k; ++j) total += chosen[j];
-        const bool divide = normalize && (score == SCORE_SIGMOID || k > 1);
+        const bool divide = normalize == 2 || (normalize && (score == SCORE_SIGMOID || k > 1));   // 2: also a single softmax pick (its weight is 1)
         for (int j = 0; j < k; ++j) weights[(size_t)r * k + j] = (divide ? chosen[j] / total : chosen[j]) * scale;
     }
 }

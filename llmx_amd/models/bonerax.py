@@ -68,8 +68,8 @@ def assemble(c: BoneraxConfig) -> ModelSpec:
                     ffn = PartSpec("dense_glu", {"hidden": E, "intermediate": layer.mlp.ff, "names": _GLU_NAMES}, p + "mlp.")
                 else:
                     ffn = PartSpec("routed_experts", {"hidden": E, "experts": layer.mlp.experts, "top_k": layer.mlp.top,
-                                                      "intermediate": layer.mlp.ff, "score": "softmax", "normalize": True, "logit_bias": True,
-                                                      "names": _EXPERT_NAMES}, p + "mlp.")
+                                                      "intermediate": layer.mlp.ff, "score": "softmax", "normalize": "always", "logit_bias": True,
+                                                      "names": _EXPERT_NAMES, "files": "per_expert"}, p + "mlp.")
             block_of[i] = len(blocks)
             blocks.append(BlockSpec(mixer_norm=norm(p + "norm1"), mixer=_mixer(c, i), ffn_norm=ffn_norm, ffn=ffn, arrangement="outnorm"))
     for i in range(len(c.layers)):

@@ -962,13 +962,15 @@ def _parts_args(z: torch.Tensor, parts: Optional[torch.Tensor]):
 def route_topk(z: torch.Tensor, bias: Optional[torch.Tensor], ids: torch.Tensor, weights: torch.Tensor, k: int, score: int,
                normalize: bool, scale: float, parts: Optional[torch.Tensor] = None, logit_bias: Optional[torch.Tensor] = None) -> None:
     """`parts` [slices, rows, experts]: the logits arrive as partial sums (gemm_f32's `parts`); they are added in slice
-    order into z first.  `logit_bias` [experts]: added to the logits (z keeps the sum) before scores are formed."""
+    order into z first.  `logit_bias` [experts]: added to the logits (z keeps the sum) before scores are formed.
+    `normalize`: False, True (the picks' weights are divided by their sum; a single softmax pick keeps its score), or
+    "always" (a single softmax pick is divided too: the softmax over the picked logits alone)."""
     rows, n_experts = z.shape
     if n_experts > MAX_EXPERTS or k > MAX_TOP_K or k > n_experts:
         raise KernelError(f"route_topk takes at most {MAX_EXPERTS} experts and {MAX_TOP_K} picks, not {n_experts} and {k}")
     _check(lib().llmx_route_topk(_dev(z, "z", torch.float32), *_parts_args(z, parts), _dev(bias, "bias", torch.float32, (n_experts,)),
                                  _dev(ids, "ids", torch.int32, (rows, k)), _dev(weights, "weights", torch.float32, (rows, k)),
-                                 rows, n_experts, k, score, 1 if normalize else 0, float(scale),
+                                 rows, n_experts, k, score, 2 if normalize == "always" else 1 if normalize else 0, float(scale),
                                  _dev(logit_bias, "logit_bias", torch.float32, (n_experts,)), _stream()), "route_topk")
 
 
@@ -1009,7 +1011,7 @@ def route_topk_align(z: torch.Tensor, bias: Optional[torch.Tensor], ids: torch.T
     """route_topk followed by moe_align; a step of at most 16 rows (sigmoid scores, at most 256 experts and 64 picks) does
     both in one launch, with the same bits."""
     rows, n_experts = z.shape
-    if score == SCORE_SIGMOID and rows <= 16 and rows * k <= 1024 and n_experts <= 256 and k <= 64 and logit_bias is None:
+    if score == SCORE_SIGMOID and rows <= 16 and rows * k <= 1024 and n_experts <= 256 and k <= 64 and logit_bias is None and normalize != "always":
         _check(lib().llmx_route_topk_align(
             _dev(z, "z", torch.float32), *_parts_args(z, parts), _dev(bias, "bias", torch.float32, (n_experts,)),
             _dev(ids, "ids", torch.int32, (rows, k)),

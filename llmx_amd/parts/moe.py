@@ -42,7 +42,7 @@ def _names(defaults: dict, given, what: str) -> dict:
 class RoutedExperts(FeedForward):
     """params: hidden, experts, top_k, intermediate, score ("sigmoid" | "softmax"), correction_bias (bool: a bias on the pick
     keys only), logit_bias (bool: a bias that is part of the router's logits), normalize (bool), scale, names ({role: name
-    below the prefix}).  score "softmax" with normalize is the softmax over the picked logits alone."""
+    below the prefix}), files ("fused" | "per_expert": how a model folder of the design holds the experts, for when no file says).  score "softmax" with normalize "always" is the softmax over the picked logits alone, for any top_k."""
     graph_safe = True
 
     wants_f32_input = True
@@ -60,7 +60,11 @@ class RoutedExperts(FeedForward):
         self.use_bias = bool(p.get("correction_bias", False))
         self.use_logit_bias = bool(p.get("logit_bias", False))
         self.names = _names(_EXPERT_NAMES, p.get("names"), "routed experts")
-        self.normalize = bool(p.get("normalize", True))
+        self.files = str(p.get("files", "fused"))
+        if self.files not in ("fused", "per_expert"):
+            raise ValueError(f"routed experts: files {self.files!r} is not one of ['fused', 'per_expert']")
+        given = p.get("normalize", True)
+        self.normalize = "always" if given == "always" else bool(given)      # "always": one softmax pick is divided by itself too
         self.scale = float(p.get("scale", 1.0))
         if not 0 < self.top_k <= self.experts:
             raise ValueError("experts per token must be between 1 and the expert count")
@@ -84,8 +88,9 @@ class RoutedExperts(FeedForward):
         has_single = any(single.match(n) for n in available)
         if has_single and fused in available:
             raise ValueError(f"{self.prefix}experts holds both fused and per-expert tensors")
-        self.per_expert = has_single
-        if has_single:
+        # a design whose files hold a tensor an expert is listed so also where no file is at hand (random weights)
+        self.per_expert = has_single or (self.files == "per_expert" and fused not in available)
+        if self.per_expert:
             # each expert's tensors go from the host straight into their places in the fused tensors
             down = nm("fused_down")
             for e in range(X):

@@ -1,0 +1,157 @@
+"""Shared by the Bonerax tests: small configurations, model folders with seeded random weights, ways of cutting a run."""
+
+from __future__ import annotations
+
+import copy
+import json
+import os
+import random
+import tempfile
+from functools import lru_cache
+
+import numpy as np
+import torch
+
+import plain_bonerax
+
+_TMP = tempfile.TemporaryDirectory(prefix="llmx_amd_bonerax_")
+
+
+def _rot(base, dims, scaling=None):
+    rot = {"base": base, "dims": dims}
+    if scaling:
+        rot["scaling"] = dict(zip(("factor", "original", "fast", "slow"), scaling))
+    return rot
+
+
+def _left(heads, kv_heads, dim, vdim, scale, window, rot):
+    return {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": scale, "mask": {"size": window}, "rot": rot}
+
+
+def _delta(heads, kv_heads, dim, vdim, conv):
+    return {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "conv": conv}
+
+
+def _moe(experts, top, ff):
+    return {"kind": "moe", "expert": {"ff": ff}, "router": {"experts": experts, "top": top}}
+
+
+def _layer(kind, mixer, mlp, weights_of=None):
+    out = {"type": kind, "mixer": mixer, "mlp": mlp}
+    if weights_of is not None:
+        out["weights_of"] = weights_of
+    return out
+
+
+_A0 = {"left": _left(4, 2, 32, 32, 0.2, 40, _rot(10000.0, 16, (4.0, 64, 16.0, 2.0))), "right": _delta(4, 2, 16, 24, 4),
+       "left_scale": 0.6, "right_scale": 1.3}
+_A1 = {"heads": 3, "dim": 16, "vdim": 40, "tau": 8.0}
+# A: sizes the matrix-core products and (keys as wide as values, pages of 16) the matrix-core attention take; shared q/k
+#    heads in both members; two layers run a second time with another layer's tensors; a layer without a feed-forward.
+CONFIG_A = {
+    "architecture": "Bonerax", "vocab": 200, "width": 96, "norm": {"eps": 1e-6}, "logit_scale": 0.7, "logit_softcap": 9.0,
+    "layers": [
+        _layer("parallel", _A0, _moe(6, 2, 48)),
+        _layer("gla", _A1, {"kind": "dense", "ff": 112}),
+        _layer("channel_delta", _delta(2, 1, 24, 16, 2), None),
+        _layer("parallel", _A0, _moe(6, 2, 48), weights_of=0),
+        _layer("gla", _A1, {"kind": "dense", "ff": 112}, weights_of=1),
+    ],
+    "ranks": {"0": {"decay": 8, "gate": 16}, "1": {"decay": 24}, "2": {"decay": 16, "gate": 8}},
+}
+# B: sizes no kernel tiles evenly (the universal products run), a window of five keys, one pick among three experts and
+#    all five of five, a convolution of one tap (no tail), one head, no soft cap.
+CONFIG_B = {
+    "architecture": "Bonerax", "vocab": 97, "width": 54, "norm": {"eps": 1e-5}, "logit_scale": 1.0,
+    "layers": [
+        _layer("channel_delta", _delta(3, 3, 5, 7, 1), _moe(3, 1, 10)),
+        _layer("parallel", {"left": _left(3, 1, 10, 6, 0.5, 5, _rot(77.0, 6)), "right": _delta(1, 1, 9, 3, 3), "left_scale": 1.0,
+                            "right_scale": 0.25}, {"kind": "dense", "ff": 21}),
+        _layer("gla", {"heads": 1, "dim": 7, "vdim": 3, "tau": 1.0}, _moe(5, 5, 6)),
+    ],
+    "ranks": {"0": {"decay": 3, "gate": 5}, "1": {"decay": 2, "gate": 1}, "2": {"decay": 4}},
+}
+# C: values wider than keys and narrower, a window no test prompt reaches, wide heads (each lane of the scan holds 32 and 64
+#    of a column's values), rotation of every dim of a head.
+CONFIG_C = {
+    "architecture": "Bonerax", "vocab": 128, "width": 64, "norm": {"eps": 1e-6}, "logit_scale": 2.0, "logit_softcap": 30.0,
+    "layers": [
+        _layer("gla", {"heads": 2, "dim": 132, "vdim": 20, "tau": 4.0}, {"kind": "dense", "ff": 64}),
+        _layer("parallel", {"left": _left(2, 2, 16, 48, 0.25, 4096, _rot(5000.0, 16, (2.0, 32, 8.0, 1.0))), "right": _delta(2, 1, 72, 8, 5),
+                            "left_scale": -0.5, "right_scale": 0.75}, _moe(4, 3, 32)),
+        _layer("parallel", {"left": _left(6, 3, 48, 16, 0.125, 17, _rot(1000.0, 8)), "right": _delta(1, 1, 8, 40, 2), "left_scale": 0.9,
+                            "right_scale": 0.9}, None),
+    ],
+    "ranks": {"0": {"decay": 8}, "1": {"decay": 16, "gate": 24}, "2": {"decay": 8, "gate": 8}},
+}
+CONFIGS = {"A": CONFIG_A, "B": CONFIG_B, "C": CONFIG_C}
+PAGES = {"A": 16, "B": 4, "C": 16}
+SEEDS = {"A": 11, "B": 12, "C": 13}
+
+
+def write_folder(config: dict, seed: int, folder: str, edit=None) -> str:
+    """A model folder of `config` with the framework's seeded random weights; `edit(tensors)` may change them first.
+    config.json is written without the low-rank projections' inner widths: a reader finds them in the tensors' shapes."""
+    from llmx_amd import RandomInit
+    from llmx_amd.models import read_config
+    from llmx_amd.weights.folder import random_tensors
+    from llmx_amd.weights.safetensors_io import write_safetensors
+    cfg = read_config(copy.deepcopy(config))
+    tensors = random_tensors(cfg, RandomInit(seed=seed, std=0.08, norm_std=0.2, bias_range=0.5, storage="bfloat16"))
+    if edit is not None:
+        edit(tensors)
+    os.makedirs(folder, exist_ok=True)
+    with open(os.path.join(folder, "config.json"), "w") as f:
+        json.dump({k: v for k, v in config.items() if k != "ranks"}, f)
+    write_safetensors(os.path.join(folder, "model.safetensors"), tensors, metadata={"format": "pt"})
+    return folder
+
+
+@lru_cache(maxsize=None)
+def model_folder(name: str) -> str:
+    return write_folder(CONFIGS[name], SEEDS[name], os.path.join(_TMP.name, name))
+
+
+def load_plain(folder: str):
+    """(config dict, {name: float64 numpy array}) of a model folder, read with the safetensors package."""
+    from safetensors.torch import load_file
+    with open(os.path.join(folder, "config.json")) as f:
+        config = json.load(f)
+    tensors = {k: v.to(torch.float64).numpy() for k, v in load_file(os.path.join(folder, "model.safetensors")).items()}
+    return config, tensors
+
+
+@lru_cache(maxsize=None)
+def plain(name: str):
+    return load_plain(model_folder(name))
+
+
+def tokens_for(name: str, length: int, seed: int):
+    rng = random.Random(104729 * seed + length)
+    return [rng.randrange(CONFIGS[name]["vocab"]) for _ in range(length)]
+
+
+@lru_cache(maxsize=None)
+def plain_logits(name: str, length: int, seed: int):
+    config, tensors = plain(name)
+    return torch.from_numpy(plain_bonerax.forward(config, tensors, tokens_for(name, length, seed)))
+
+
+def greedy(config, tensors, prompt, n):
+    """n tokens, each the largest logit after everything before it (the whole sequence is run again for each)."""
+    seq = list(prompt)
+    for _ in range(n):
+        seq.append(int(np.argmax(plain_bonerax.forward(config, tensors, seq)[-1])))
+    return seq[len(prompt):]
+
+
+def portions(length: int, seed: int, smallest: int = 2):
+    """Cuts [0, length) into portions of changing size, several of them of `smallest` tokens."""
+    rng = random.Random(seed)
+    cuts, at = [], 0
+    sizes = [smallest, 7, smallest, 16, 3, 33, smallest, 64, 5]
+    while at < length:
+        n = min(length - at, sizes[len(cuts) % len(sizes)] if rng.random() < 0.7 else rng.randrange(1, 40))
+        cuts.append((at, at + n))
+        at += n
+    return cuts

@@ -181,13 +181,15 @@ def glu(h, gate, up, down):
     return (silu(h @ gate.T) * (h @ up.T)) @ down.T
 
 
-def routed_experts(h, w, mlp, picks_out=None):
-    """w: router, router.b, e<i>.gate / up / down.  The `top` largest logits pick; weights are their softmax."""
+def routed_experts(h, w, mlp, picks_out=None, picks_in=None):
+    """w: router, router.b, e<i>.gate / up / down.  The `top` largest logits pick; weights are their softmax.
+    `picks_in` [T, top] replaces the choice (not the weights): a comparison with an implementation that rounds elsewhere
+    hands its picks over, so that a near tie that fell the other way does not count as a difference."""
     z = h @ w["router"].T + w["router.b"]
     top = mlp["router"]["top"]
     out = np.zeros_like(h)
     for t in range(h.shape[0]):
-        ids = sorted(range(z.shape[1]), key=lambda e: (-z[t, e], e))[:top]
+        ids = sorted(range(z.shape[1]), key=lambda e: (-z[t, e], e))[:top] if picks_in is None else [int(e) for e in picks_in[t]]
         p = np.exp(z[t, ids] - z[t, ids].max())
         p /= p.sum()
         if picks_out is not None:
@@ -202,8 +204,10 @@ def under(tensors, prefix):
     return {k[len(prefix):]: np.asarray(v, dtype=np.float64) for k, v in tensors.items() if k.startswith(prefix)}
 
 
-def forward(config, tensors, tokens, residuals=None):
-    """Logits [T, vocab] of one sequence.  `residuals`, a list, receives x after every layer run."""
+def forward(config, tensors, tokens, residuals=None, picks=None):
+    """Logits [T, vocab] of one sequence.  `residuals`, a list, receives x after every layer run; `picks`, a list with one
+    [T, top] array for every routed layer run in order, replaces the routers' choices."""
+    picks = list(picks) if picks is not None else None
     eps = config["norm"]["eps"]
     x = np.asarray(tensors["embed"], dtype=np.float64)[np.asarray(tokens)]
     for i, layer in enumerate(config["layers"]):
@@ -223,7 +227,10 @@ def forward(config, tensors, tokens, residuals=None):
         mlp = layer.get("mlp")
         if mlp is not None:
             ff = under(tensors, p + "mlp.")
-            y = glu(x, ff["gate"], ff["up"], ff["down"]) if mlp["kind"] == "dense" else routed_experts(x, ff, mlp)
+            if mlp["kind"] == "dense":
+                y = glu(x, ff["gate"], ff["up"], ff["down"])
+            else:
+                y = routed_experts(x, ff, mlp, picks_in=picks.pop(0) if picks is not None else None)
             x = x + layer_norm(y, np.asarray(tensors[p + "norm2"], dtype=np.float64), eps)
         if residuals is not None:
             residuals.append(x.copy())
