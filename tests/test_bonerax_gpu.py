@@ -29,7 +29,7 @@ pytestmark = pytest.mark.gpu
 
 F32_TOL = 3e-5      # |engine - plain| over all logits relative to the largest |logit|: float32 sums in another order
 BF16_TOL = 4e-2     # the serving path against the plain implementation (float64, nothing rounded), with the engine's expert picks
-BF16_RMS = 1.5e-2   # ... and the root mean square of all differences relative to that of the logits
+BF16_RMS = 2.5e-2   # ... and the root mean square of all differences relative to that of the logits
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
