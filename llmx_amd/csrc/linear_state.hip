@@ -3,8 +3,8 @@
 //     S <- diag(g_t) S                         (a decay a key channel, acting on S's rows)
 //     u  = beta_t (v_t - S^T k_t)              (delta rule; without it u = v_t: gated linear attention)
 //     S <- S + k_t u^T,   o_t = S^T q_t        (the read-out sees the token's own write)
-// A column of S (one value channel) never meets another, so the scan gives every column to four lanes that hold a quarter
-// of its D values each in registers and walk a request's rows in order: the state after a row is the same bits however
+// A column of S (one value channel) never meets another, so the scan gives every column to sixteen lanes that hold a
+// sixteenth of its D values each in registers and walk a request's rows in order: the state after a row is the same bits however
 // the rows were cut into steps.  Decays, gates, unit norms and the state are float32 in both number formats.
 // Around it: the preparation of a delta-rule row (short causal convolutions with silu, unit-norm q and k, the decay and
 // beta), the decay of gated linear attention, and the gated RMS norm of the read-out.
@@ -107,10 +107,10 @@ extern "C" int llmx_sigmoid_root(const float* z, const float* bias, float inv_ta
 }
 
 // ---------------------------------------------------------------------------
-// The scan.  Grid (H * ceil(V / 16), entries), one wave a block: lane = 16 s + c owns value channel 16 * tile + c and
-// key channels [s R, s R + R) of its head.  q and k are read head h / share (several heads may share one), with row
-// strides of their own, so they may be columns of a wider projection.  The next row's operands are asked for before this
-// row is worked on.  Sums over a column's four lanes: (s0 + s1) + (s2 + s3).
+// The scan.  Grid (H * ceil(V / 8), entries), two waves a block: the 16 lanes of a row of lanes own value channel
+// 8 * tile + c together, lane s of them the key channels [s R, s R + R) of its head.  q and k are read head h / share (several heads may share one), with row
+// strides of their own, so they may be columns of a wider projection.  A lane's sums over its R channels run in up to four
+// chains (channels i, i + 4, ...: (c0 + c1) + (c2 + c3)); sums over a column's sixteen lanes are a butterfly over the row.
 // The block of tile 0 of an entry also hands on the convolution tail: the entry's last taps - 1 inputs, from this step's
 // rows of `tail_src` and, where the step brought fewer, from the old tail.
 struct StateScanArgs {
@@ -132,14 +132,35 @@ struct StateScanArgs {
     int tail_ld, tail_C, taps, tail_off;
 };
 
-template <int R, bool AHEAD>
-__global__ void __launch_bounds__(64) state_scan_kernel(StateScanArgs a) {
-    const int lane = threadIdx.x, s = lane >> 4, c = lane & 15;
-    const int tiles = (a.V + 15) / 16;
+// Rows are worked on in chunks of CH: the block brings a chunk's q, k and decay values (its head's D of each, padded to
+// 16 R) and its 8 values of v and beta through registers into LDS while the chunk before is worked on, so the chain from
+// token to token waits for LDS, not for memory; a token's operands are read from LDS while the token before is worked on.
+// Every load is asked for whatever the index (addresses are clamped, the value is chosen afterwards), so none sits behind
+// a branch.
+__device__ __forceinline__ float row16_sum(float v) {      // the sum over a row of 16 lanes, the same bits in each
+    v += row_rotate<8>(v);
+    v += row_rotate<4>(v);
+    v += row_rotate<2>(v);
+    v += row_rotate<1>(v);
+    return v;
+}
+
+#define SCAN_COLS 8     // value channels a block of two waves owns
+template <int R, int CH>
+__global__ void __launch_bounds__(128) state_scan_kernel(StateScanArgs a) {
+    constexpr int DP = 16 * R;                      // a head's key channels, padded
+    constexpr int PER_TOKEN = 3 * DP;               // k | q | decay
+    constexpr int STAGE = (CH * PER_TOKEN + 127) / 128;   // values a thread brings a chunk
+    constexpr int NC = R >= 4 ? 4 : R;              // chains a lane's sums run in
+    __shared__ __attribute__((aligned(16))) float rows[2][CH][PER_TOKEN];
+    __shared__ float vals[2][CH][SCAN_COLS];
+    __shared__ float betas[2][CH];
+    const int tid = threadIdx.x, lane = tid & 63, s = lane & 15, c = (tid >> 4);     // c: 0..7, the block's column
+    const int tiles = (a.V + SCAN_COLS - 1) / SCAN_COLS;
     const int h = blockIdx.x / tiles, tile = blockIdx.x % tiles;
     const int e = blockIdx.y;
     const int row0 = a.entry_rows[2 * e], n = a.entry_rows[2 * e + 1];
-    const int j = tile * 16 + c;
+    const int j = tile * SCAN_COLS + c;
     const bool col = j < a.V;
     const int d0 = s * R;
     const size_t slot_r = (size_t)a.slot_read[e] * a.state_stride, slot_w = (size_t)a.slot_write[e] * a.state_stride;
@@ -147,7 +168,7 @@ __global__ void __launch_bounds__(64) state_scan_kernel(StateScanArgs a) {
     if (a.taps > 1 && blockIdx.x == 0) {
         const float* old = a.state + slot_r + a.tail_off;
         float* fresh = a.state + slot_w + a.tail_off;
-        for (int ch = lane; ch < a.tail_C; ch += 64) {
+        for (int ch = tid; ch < a.tail_C; ch += 128) {
             for (int p = 0; p < a.taps - 1; ++p) {      // ascending: in place, a value is read before its place is written
                 const int idx = n - (a.taps - 1) + p;
                 fresh[(size_t)p * a.tail_C + ch] = idx >= 0 ? a.tail_src[(size_t)(row0 + idx) * a.tail_ld + ch] : old[(size_t)(n + p) * a.tail_C + ch];
@@ -155,65 +176,105 @@ __global__ void __launch_bounds__(64) state_scan_kernel(StateScanArgs a) {
         }
     }
 
+    const int hq = h / a.share;
+    const float* kp = a.k + (size_t)hq * a.D;
+    const float* qp = a.q + (size_t)hq * a.D;
+    const float* gp = a.decay + (size_t)h * a.D;
+    const float* vp = a.v + (size_t)h * a.V + tile * SCAN_COLS;
+    float stage[STAGE], vstage = 0.0f, bstage = 0.0f;
+    auto fetch = [&](int t0) {
+#pragma unroll
+        for (int u = 0; u < STAGE; ++u) {
+            const int idx = min(tid + 128 * u, CH * PER_TOKEN - 1);
+            const int tt = idx / PER_TOKEN, rem = idx % PER_TOKEN, which = rem / DP, d = rem % DP;
+            const size_t row = (size_t)(row0 + min(t0 + tt, n - 1));
+            const int dd = d < a.D ? d : 0;
+            const float* src = which == 0 ? kp + row * a.ldk : which == 1 ? qp + row * a.ldq : gp + row * a.ldg;
+            const float x = src[dd];
+            stage[u] = d < a.D ? x : 0.0f;
+        }
+        if (CH * SCAN_COLS <= 128 || tid < CH * SCAN_COLS) {
+            const int tt = min(tid / SCAN_COLS, CH - 1), cc = tid % SCAN_COLS;
+            vstage = vp[(size_t)(row0 + min(t0 + tt, n - 1)) * a.ldv + min(cc, a.V - 1 - tile * SCAN_COLS)];
+        }
+        if (a.beta) bstage = a.beta[(size_t)(row0 + min(t0 + min(tid, CH - 1), n - 1)) * a.H + h];
+    };
+    auto put = [&](int b) {
+#pragma unroll
+        for (int u = 0; u < STAGE; ++u)
+            if (tid + 128 * u < CH * PER_TOKEN) (&rows[b][0][0])[tid + 128 * u] = stage[u];
+        if (tid < CH * SCAN_COLS) (&vals[b][0][0])[tid] = vstage;
+        if (tid < CH) betas[b][tid] = bstage;
+    };
+
+    fetch(0);
     float S[R];
     {
-        const float* src = a.state + slot_r + ((size_t)h * a.D) * a.V + j;
+        const float* src = a.state + slot_r + ((size_t)h * a.D) * a.V + (col ? j : 0);
 #pragma unroll
-        for (int i = 0; i < R; ++i) S[i] = (col && d0 + i < a.D) ? src[(size_t)(d0 + i) * a.V] : 0.0f;
+        for (int i = 0; i < R; ++i) {
+            const float x = src[(size_t)(d0 + i < a.D ? d0 + i : 0) * a.V];
+            S[i] = (col && d0 + i < a.D) ? x : 0.0f;
+        }
     }
-    const int hq = h / a.share;
-    const float* qp = a.q + (size_t)hq * a.D;
-    const float* kp = a.k + (size_t)hq * a.D;
-    const float* gp = a.decay + (size_t)h * a.D;
-    const float* vp = a.v + (size_t)h * a.V + (col ? j : 0);
-    float nk[R], nq[R], ng[R], nv, nb = 0.0f;
-    auto fetch = [&](int t) {
-        const size_t row = (size_t)(row0 + t);
+    put(0);
+    __syncthreads();
+    const bool delta = a.beta != nullptr;
+    float nk[R], nq[R], ng[R], nv, nb;
+    auto read = [&](int b, int tt) {
+        const float* kr = &rows[b][tt][d0];
 #pragma unroll
         for (int i = 0; i < R; ++i) {
-            const bool in = d0 + i < a.D;
-            const int d = in ? d0 + i : 0;
-            const float kv = kp[row * a.ldk + d], qv = qp[row * a.ldq + d], gv = gp[row * a.ldg + d];
-            nk[i] = in ? kv : 0.0f;
-            nq[i] = in ? qv : 0.0f;
-            ng[i] = in ? gv : 0.0f;
+            nk[i] = kr[i];
+            nq[i] = kr[DP + i];
+            ng[i] = kr[2 * DP + i];
         }
-        nv = vp[row * a.ldv];
-        if (a.beta) nb = a.beta[row * a.H + h];
+        nv = vals[b][tt][c];
+        nb = betas[b][tt];
     };
-    if (AHEAD) fetch(0);
-    for (int t = 0; t < n; ++t) {
-        if (!AHEAD) fetch(t);      // a quarter column of 64 values leaves no registers for a second set of operands
-        float ck[R], cq[R], cg[R];
-#pragma unroll
-        for (int i = 0; i < R; ++i) {
-            ck[i] = nk[i];
-            cq[i] = nq[i];
-            cg[i] = ng[i];
-        }
-        const float cv = nv, cb = nb;
-        if (AHEAD) fetch(t + 1 < n ? t + 1 : n - 1);
-        float u = cv;
-        if (a.beta) {
-            float p = 0.0f;
+    for (int t0 = 0, b = 0; t0 < n; t0 += CH, b ^= 1) {
+        fetch(t0 + CH);             // past the end the last row is asked for again and never used
+        const int m = min(CH, n - t0);
+        read(b, 0);
+        for (int tt = 0; tt < m; ++tt) {
+            float ck[R], cq[R], cg[R];
 #pragma unroll
             for (int i = 0; i < R; ++i) {
-                S[i] = S[i] * cg[i];
-                p = fmaf(ck[i], S[i], p);
+                ck[i] = nk[i];
+                cq[i] = nq[i];
+                cg[i] = ng[i];
             }
-            u = cb * (cv - rows_sum4(p));
-        } else {
+            float u = nv;
+            const float cb = nb;
+            read(b, tt + 1 < CH ? tt + 1 : tt);
+            if (delta) {
+                float p[NC];
 #pragma unroll
-            for (int i = 0; i < R; ++i) S[i] = S[i] * cg[i];
-        }
-        float o = 0.0f;
+                for (int x = 0; x < NC; ++x) p[x] = 0.0f;
 #pragma unroll
-        for (int i = 0; i < R; ++i) {
-            S[i] = fmaf(ck[i], u, S[i]);
-            o = fmaf(cq[i], S[i], o);
+                for (int i = 0; i < R; ++i) {
+                    S[i] = S[i] * cg[i];
+                    p[i % NC] = fmaf(ck[i], S[i], p[i % NC]);
+                }
+                const float dot = NC == 4 ? (p[0] + p[1]) + (p[2] + p[3]) : NC == 2 ? p[0] + p[1] : p[0];
+                u = cb * (u - row16_sum(dot));
+            } else {
+#pragma unroll
+                for (int i = 0; i < R; ++i) S[i] = S[i] * cg[i];
+            }
+            float o[NC];
+#pragma unroll
+            for (int x = 0; x < NC; ++x) o[x] = 0.0f;
+#pragma unroll
+            for (int i = 0; i < R; ++i) {
+                S[i] = fmaf(ck[i], u, S[i]);
+                o[i % NC] = fmaf(cq[i], S[i], o[i % NC]);
+            }
+            const float sum = row16_sum(NC == 4 ? (o[0] + o[1]) + (o[2] + o[3]) : NC == 2 ? o[0] + o[1] : o[0]);
+            if (s == 0 && col) a.out[(size_t)(row0 + t0 + tt) * a.H * a.V + (size_t)h * a.V + j] = sum * a.out_scale;
         }
-        o = rows_sum4(o);
-        if (s == 0 && col) a.out[(size_t)(row0 + t) * a.H * a.V + (size_t)h * a.V + j] = o * a.out_scale;
+        put(b ^ 1);
+        __syncthreads();
     }
     {
         float* dst = a.state + slot_w + ((size_t)h * a.D) * a.V + j;
@@ -231,13 +292,14 @@ extern "C" int llmx_state_scan(const float* q, int ldq, const float* k, int ldk,
     if (H < 1 || share < 1 || H % share || D < 1 || D > 256 || V < 1 || (taps > 1 && !tail_src)) return -2;
     StateScanArgs a{q, k, v, decay, beta, ldq, ldk, ldv, ldg, state, state_stride, slot_read, slot_write, entry_rows, out, out_scale,
                     H, share, D, V, tail_src, tail_ld, tail_C, taps, tail_off};
-    const dim3 grid((unsigned)(H * ((V + 15) / 16)), (unsigned)n_entries);
+    const dim3 grid((unsigned)(H * ((V + SCAN_COLS - 1) / SCAN_COLS)), (unsigned)n_entries);
     llmx_note_launch(LK_STATE_SCAN);
-    const int per_lane = (D + 3) / 4;
-    if (per_lane <= 8) hipLaunchKernelGGL((state_scan_kernel<8, true>), grid, dim3(64), 0, stream, a);
-    else if (per_lane <= 16) hipLaunchKernelGGL((state_scan_kernel<16, true>), grid, dim3(64), 0, stream, a);
-    else if (per_lane <= 32) hipLaunchKernelGGL((state_scan_kernel<32, true>), grid, dim3(64), 0, stream, a);
-    else hipLaunchKernelGGL((state_scan_kernel<64, false>), grid, dim3(64), 0, stream, a);
+    const int per_lane = (D + 15) / 16;
+    if (per_lane <= 1) hipLaunchKernelGGL((state_scan_kernel<1, 8>), grid, dim3(128), 0, stream, a);
+    else if (per_lane <= 2) hipLaunchKernelGGL((state_scan_kernel<2, 8>), grid, dim3(128), 0, stream, a);
+    else if (per_lane <= 4) hipLaunchKernelGGL((state_scan_kernel<4, 8>), grid, dim3(128), 0, stream, a);
+    else if (per_lane <= 8) hipLaunchKernelGGL((state_scan_kernel<8, 8>), grid, dim3(128), 0, stream, a);
+    else hipLaunchKernelGGL((state_scan_kernel<16, 8>), grid, dim3(128), 0, stream, a);
     return LLMX_CHECK_LAUNCH();
 }
 

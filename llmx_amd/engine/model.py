@@ -33,6 +33,13 @@ class BuiltModel:
         for b in self.blocks:
             out.extend(b.parts())
         out += [self.final_norm, self.head]
+        # a part made of parts (mixers side by side) is followed by its members, which list and take their own tensors
+        at = 0
+        while at < len(out):
+            members = getattr(out[at], "members", None)
+            if members is not None:
+                out[at + 1:at + 1] = list(members())
+            at += 1
         return out
 
     def tensor_specs(self, available: Set[str] = frozenset()) -> List[TensorSpec]:

@@ -18,7 +18,8 @@ from .spec import CompositeNeed, PartSpec
 
 class SideBySide(Mixer):
     """params: hidden; members: a list of {name, scale, mixer (PartSpec)}.  A member's tensors start with its own prefix
-    (its PartSpec's)."""
+    (its PartSpec's); a built model lists the members as parts of their own after this one (`members()`), so each names
+    and takes its tensors and has its say in a recorded step's key itself."""
 
     steps_between_slots = True      # every member with state says so itself; the engine asks the members
 
@@ -39,16 +40,6 @@ class SideBySide(Mixer):
 
     def cache_need(self):
         return CompositeNeed(tuple(m.cache_need() for m in self._members))
-
-    def tensor_specs(self, available):
-        return [s for m in self._members for s in m.tensor_specs(available)]
-
-    def load(self, tensors):
-        for m in self._members:
-            m.load(tensors)
-
-    def graph_key(self, step):
-        return tuple(m.graph_key(step) for m in self._members)
 
     def forward(self, step, h, out, accumulate, cache: LayerCache, h32=None):
         T = step.rows

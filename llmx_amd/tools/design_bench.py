@@ -1,5 +1,9 @@
 """Prefill and decode throughput of one design beside the closest other one at equal size, with random weights.
 
+`python bench.py --design bonerax` does the same for a Bonerax (layers in turn: windowed attention beside a delta rule,
+gated linear attention, the delta rule alone; routed SwiGLU experts) and a MiniMax-M3 with the same width, layers, heads,
+head width and experts.
+
 `python bench.py --design nenotar` measures, at sizes that resemble a real model's layers, a Nenotar (latent attention
 and minGRU layers in turn, each with a dense xIELU feed-forward and a per-layer token input) and a MiniMax-M3 of the
 same width, layers, heads and vocabulary whose routed experts hold the same active weights a token: one 2,048-token
@@ -48,6 +52,47 @@ def closest_config(width, layers, heads, ff, recurrent, side, vocab):
                            max_position_embeddings=2 * CONTEXT)
 
 
+# name -> (width, layers, attention heads, kv heads, window, recurrent heads (of 128 x 128), experts, picks, expert ff, vocab)
+BONERAX_SIZES = {
+    "w2048": (2048, 6, 16, 4, 1024, 16, 8, 2, 2048, 32768),
+    "w4096": (4096, 3, 32, 8, 1024, 32, 8, 2, 4096, 32768),
+    "w256": (256, 3, 2, 1, 64, 2, 4, 2, 128, 1024),
+}
+
+
+def bonerax_config(width, layers, heads, kv_heads, window, rec_heads, experts, top, ff, vocab):
+    from llmx_amd.config.bonerax import (BoneraxConfig, DeltaConfig, GLAConfig, LayerConfig, MLPConfig, ParallelConfig, RotaryScaling,
+                                         WindowAttentionConfig)
+    left = WindowAttentionConfig(heads=heads, kv_heads=kv_heads, dim=128, vdim=128, scale=128 ** -0.5, window=window, rot_base=10000.0,
+                                 rot_dims=64, rot_scaling=RotaryScaling(8.0, 4096.0, 32.0, 1.0))
+    delta = DeltaConfig(heads=rec_heads, kv_heads=rec_heads, dim=128, vdim=128, conv=4)
+    kinds = [("parallel", ParallelConfig(left, DeltaConfig(heads=max(1, rec_heads // 4), kv_heads=max(1, rec_heads // 4), dim=128, vdim=128, conv=4),
+                                         0.8, 0.9)),
+             ("gla", GLAConfig(heads=rec_heads, dim=64, vdim=128, tau=16.0)), ("channel_delta", delta)]
+    mlp = MLPConfig("moe", ff, experts=experts, top=top)
+    rank = max(16, width // 32)
+    return BoneraxConfig(vocab=vocab, width=width, norm_eps=1e-5, logit_scale=1.0, logit_softcap=30.0,
+                         layers=tuple(LayerConfig(*kinds[i % 3], mlp) for i in range(layers)),
+                         ranks={i: {"decay": rank, "gate": rank} for i in range(layers)})
+
+
+def bonerax_closest(width, layers, heads, kv_heads, window, rec_heads, experts, top, ff, vocab):
+    """MiniMax-M3 of the same width, layers, heads, head width, experts, picks and expert width."""
+    from llmx_amd import MiniMaxM3Config
+    return MiniMaxM3Config(vocab_size=vocab, hidden_size=width, num_hidden_layers=layers, num_attention_heads=heads, num_key_value_heads=kv_heads,
+                           head_dim=128, rotary_dim=64, rope_theta=1e6, rms_norm_eps=1e-6, num_local_experts=experts, num_experts_per_tok=top,
+                           intermediate_size=ff, routed_scaling_factor=1.0, norm_topk_prob=True, tie_word_embeddings=False,
+                           max_position_embeddings=2 * CONTEXT)
+
+
+def _layer_mixers(layer):
+    """(windowed attention or None, [recurrences as (heads, dim, vdim, delta?)]) of a Bonerax layer."""
+    m = layer.mixer
+    if layer.type == "parallel":
+        return m.left, [(m.right.heads, m.right.dim, m.right.vdim, True)]
+    return None, [(m.heads, m.dim, m.vdim, layer.type == "channel_delta")]
+
+
 def _ids(n, vocab, seed):
     x, out = (seed * 2654435761 + 1) & 0xFFFFFFFF, []
     for _ in range(n):
@@ -62,6 +107,16 @@ def cache_bytes_a_token(engine) -> int:
                for arenas in engine._paged for t in arenas.values())
 
 
+def cache_bytes_read(engine, context: float) -> float:
+    """Bytes of cache and state a decoded token of one request at `context` tokens must read (and, for states, write):
+    a windowed group's keys and values only as far as the window reaches."""
+    total = 0.0
+    for need, arenas in zip(engine.group_needs, engine._paged):
+        tokens = min(context, need.window) if need.window else context
+        total += tokens * sum(t.shape[0] * (t.numel() // (t.shape[0] * t.shape[1]) // engine.page_tokens) * t.element_size() for t in arenas.values())
+    return total + 2 * sum(t[0].numel() * t.element_size() for t in engine._state)
+
+
 def prompt_flops(engine, T) -> float:
     """Multiply-adds x 2 of a T-token prompt: every weight matrix once a row (the head for one row), and the attention
     layers' score and value products over the causal half."""
@@ -74,6 +129,17 @@ def prompt_flops(engine, T) -> float:
         expert = 3 * cfg.hidden_size * cfg.intermediate_size
         dense -= 2.0 * T * cfg.num_hidden_layers * (cfg.num_local_experts - cfg.num_experts_per_tok) * expert
         attn = cfg.num_hidden_layers * 4.0 * cfg.num_attention_heads * cfg.head_dim * T * (T + 1) / 2
+    elif cfg.architecture == "Bonerax":
+        attn = 0.0
+        for layer in cfg.layers:
+            if layer.mlp is not None and layer.mlp.kind == "moe":
+                dense -= 2.0 * T * (layer.mlp.experts - layer.mlp.top) * 3 * cfg.width * layer.mlp.ff
+            left, recurrences = _layer_mixers(layer)
+            if left is not None:
+                keys = sum(min(t + 1, left.window) for t in range(T))
+                attn += 2.0 * left.heads * (left.dim + left.vdim) * keys
+            for heads, dim, vdim, delta in recurrences:      # decay, (S^T k,) the outer product, S^T q: a token a head
+                attn += T * heads * dim * vdim * (2.0 * (3 if delta else 2) + 1.0)
     else:
         attn = 0.0
         for layer in cfg.layers:
@@ -135,11 +201,15 @@ def measure(engine, torch, steps, warmup):
         dt = (time.perf_counter() - t0) / steps
         for rid in rids:
             engine.end_request(rid)
-        need = engine.weight_bytes() + batch * (CONTEXT - steps / 2) * cache_bytes_a_token(engine)
+        need = engine.weight_bytes() + batch * cache_bytes_read(engine, CONTEXT - steps / 2)
         cfg = engine.config
         if hasattr(cfg, "num_local_experts"):   # of the experts at most batch x picks are read
             unread = max(0, cfg.num_local_experts - batch * cfg.num_experts_per_tok)
             need -= cfg.num_hidden_layers * unread * 3 * cfg.hidden_size * cfg.intermediate_size * 2
+        elif cfg.architecture == "Bonerax":
+            for layer in cfg.layers:
+                if layer.mlp is not None and layer.mlp.kind == "moe":
+                    need -= max(0, layer.mlp.experts - batch * layer.mlp.top) * 3 * cfg.width * layer.mlp.ff * 2
         side = getattr(cfg, "token_side_dim", None) or 0
         need -= 2 * vocab * side * (len(cfg.layers) if side else 0)     # of the token table a step reads its rows only
         need -= 2 * vocab * engine.spec.hidden_size                     # and of the embedding
@@ -148,19 +218,26 @@ def measure(engine, torch, steps, warmup):
     return rec
 
 
+DESIGNS = {
+    "nenotar": ("Nenotar", "MiniMax-M3 (GQA attention, routed SwiGLU experts)", SIZES, nenotar_config, closest_config),
+    "bonerax": ("Bonerax", "MiniMax-M3 (GQA attention, routed SwiGLU experts)", BONERAX_SIZES, bonerax_config, bonerax_closest),
+}
+
+
 def run(design: str, steps: int, warmup: int, sizes=None) -> dict:
     import torch
     from llmx_amd import Engine, RandomInit
-    if design != "nenotar":
-        raise SystemExit(f"bench: no design named {design!r} (known: nenotar)")
-    result = {"design": "Nenotar", "closest": "MiniMax-M3 (GQA attention, routed SwiGLU experts)", "dtype": "bf16", "prompt": PROMPT,
+    if design not in DESIGNS:
+        raise SystemExit(f"bench: no design named {design!r} (known: {sorted(DESIGNS)})")
+    title, closest, table, make_design, make_closest = DESIGNS[design]
+    result = {"design": title, "closest": closest, "dtype": "bf16", "prompt": PROMPT,
               "context": CONTEXT, "data": "synthetic: LCG token ids, N(0,0.02) weights generated on the device", "sizes": {}}
     for name in (sizes or DEFAULT_SIZES):
-        if name not in SIZES:
-            raise SystemExit(f"bench: no size named {name!r} (known: {sorted(SIZES)})")
-        shape = SIZES[name]
+        if name not in table:
+            raise SystemExit(f"bench: no size named {name!r} (known: {sorted(table)})")
+        shape = table[name]
         per = {}
-        for which, make in (("nenotar", nenotar_config), ("closest", closest_config)):
+        for which, make in ((design, make_design), ("closest", make_closest)):
             engine = Engine.from_random(make(*shape), RandomInit(seed=0, std=0.02), dtype="bfloat16", kv_tokens=8 * CONTEXT + 4 * PROMPT,
                                         page_tokens=16, max_requests=8)
             per[which] = measure(engine, torch, steps, max(2, warmup))
