@@ -162,6 +162,26 @@ extern "C" int llmx_cast_rows(const float* x, void* out, int out_dtype, long tot
     return LLMX_CHECK_LAUNCH();
 }
 
+// out[t, :] = x[t, col0 : col0 + n] in the activation type: some columns of a wider float32 projection as the rows a further
+// product reads (the inner values of a low-rank projection).
+template <typename TO>
+__global__ void __launch_bounds__(256) cast_cols_kernel(const float* __restrict__ x, int ld, TO* __restrict__ out, int n, size_t total) {
+    const size_t at = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (at >= total) return;
+    st(out + at, x[(at / (size_t)n) * (size_t)ld + (at % (size_t)n)]);
+}
+
+extern "C" int llmx_cast_cols(const float* x, int ld, void* out, int out_dtype, int rows, int n, hipStream_t stream) {
+    if (rows <= 0 || n <= 0) return 0;
+    if (ld < n) return -2;
+    llmx_note_launch(LK_CAST_ROWS);
+    const size_t total = (size_t)rows * n;
+    const dim3 grid((unsigned)((total + 255) / 256));
+    if (out_dtype == LLMX_F32) hipLaunchKernelGGL(cast_cols_kernel<float>, grid, dim3(256), 0, stream, x, ld, (float*)out, n, total);
+    else hipLaunchKernelGGL(cast_cols_kernel<bf16_t>, grid, dim3(256), 0, stream, x, ld, (bf16_t*)out, n, total);
+    return LLMX_CHECK_LAUNCH();
+}
+
 // out (=, +=) sa * (a + bias_a) + sb * b over float32 rows [T, n]: the join of mixers that run side by side, and a
 // projection's bias; bias_a and b may be null.
 __global__ void __launch_bounds__(256) combine_rows_kernel(float* __restrict__ out, const float* __restrict__ a, float sa,

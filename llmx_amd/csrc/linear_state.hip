@@ -13,7 +13,7 @@
 __device__ __forceinline__ float sigmoid_ls(float v) { return 1.0f / (1.0f + expf(-v)); }
 
 // ---------------------------------------------------------------------------
-// One block a row.  The fused in-projection's row `pre` holds q (G*D) | k (G*D) | v (H*V) at its start and beta's H
+// The fused in-projection's row `pre` holds q (G*D) | k (G*D) | v (H*V) at its start and beta's H
 // pre-activations at `beta_col`.  Channel c of q | k | v passes a causal convolution over the request's last `taps`
 // inputs (weights [C, taps], the last column weighs the row itself): inputs of earlier steps come from the tail the state
 // slot keeps ([taps - 1, C] at `tail_off`, oldest first; zero when the request opened), inputs of this step from `pre`.
@@ -22,7 +22,8 @@ struct DeltaPrepArgs {
     const float* pre;
     int ld;
     const float* conv_w;
-    const float* step_pre;   // [T, H*D]: the decay's projection before its bias
+    const float* step_pre;   // [T, H*D] (rows step_ld apart): the decay's projection before its bias
+    int step_ld;
     const float* dt_bias;    // [H*D]
     const float* a_log;      // [H]
     const float* state;
@@ -39,52 +40,68 @@ struct DeltaPrepArgs {
     int G, H, D, V, taps, beta_col;
 };
 
-__global__ void __launch_bounds__(256) delta_prep_kernel(DeltaPrepArgs a) {
-    extern __shared__ float chan[];
-    const int t = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+// One wave a (row, unit): the units of a row are its 2 G heads of q and k (convolution, silu, unit norm), its H heads of
+// v (convolution, silu), its H heads of decays, and beta; a unit's values stay in the wave's registers.
+#define PREP_MAX 256     // values of a head a wave keeps (4 a lane): the scan's limit on a head's key channels
+__device__ __forceinline__ float conv_silu_at(const DeltaPrepArgs& a, const float* __restrict__ tail, int C, int row0, int i, int c) {
+    float acc = 0.0f;
+    for (int j = 0; j < a.taps; ++j) {
+        const int idx = i - (a.taps - 1) + j;
+        const float x = idx >= 0 ? a.pre[(size_t)(row0 + idx) * a.ld + c] : tail[(size_t)(a.taps - 1 + idx) * C + c];
+        acc = fmaf(a.conv_w[(size_t)c * a.taps + j], x, acc);
+    }
+    return acc * sigmoid_ls(acc);
+}
+
+__global__ void __launch_bounds__(64) delta_prep_kernel(DeltaPrepArgs a) {
+    const int t = blockIdx.x, unit = blockIdx.y, lane = threadIdx.x;
     const int GD = a.G * a.D, HV = a.H * a.V, HD = a.H * a.D;
     const int C = 2 * GD + HV;
     const int e = a.row_entry[t];
     const int row0 = a.entry_rows[2 * e];
     const int i = t - row0;
     const float* tail = a.state + (size_t)a.slot_read[e] * a.state_stride + a.tail_off;
-    for (int c = tid; c < C; c += 256) {
-        float acc = 0.0f;
-        for (int j = 0; j < a.taps; ++j) {
-            const int idx = i - (a.taps - 1) + j;
-            const float x = idx >= 0 ? a.pre[(size_t)(row0 + idx) * a.ld + c] : tail[(size_t)(a.taps - 1 + idx) * C + c];
-            acc = fmaf(a.conv_w[(size_t)c * a.taps + j], x, acc);
-        }
-        chan[c] = acc * sigmoid_ls(acc);
-    }
-    __syncthreads();
-    for (int hh = wave; hh < 2 * a.G; hh += 4) {
-        const float* head = chan + (size_t)hh * a.D;
+    if (unit < 2 * a.G) {                               // a head of q or k
+        const int c0 = unit * a.D;
+        float y[PREP_MAX / 64];
         float ss = 0.0f;
-        for (int d = lane; d < a.D; d += 64) ss = fmaf(head[d], head[d], ss);
+#pragma unroll
+        for (int u = 0; u < PREP_MAX / 64; ++u) {
+            const int d = lane + 64 * u;
+            y[u] = d < a.D ? conv_silu_at(a, tail, C, row0, i, c0 + d) : 0.0f;
+            ss = fmaf(y[u], y[u], ss);
+        }
         const float r = 1.0f / sqrtf(wave_sum(ss) + 1e-6f);
-        float* out = (hh < a.G ? a.q + (size_t)t * GD + (size_t)hh * a.D : a.k + (size_t)t * GD + (size_t)(hh - a.G) * a.D);
-        for (int d = lane; d < a.D; d += 64) out[d] = head[d] * r;
+        float* out = unit < a.G ? a.q + (size_t)t * GD + c0 : a.k + (size_t)t * GD + (c0 - GD);
+#pragma unroll
+        for (int u = 0; u < PREP_MAX / 64; ++u)
+            if (lane + 64 * u < a.D) out[lane + 64 * u] = y[u] * r;
+    } else if (unit < 2 * a.G + a.H) {                  // a head of v
+        const int h = unit - 2 * a.G;
+        for (int d = lane; d < a.V; d += 64) a.v[(size_t)t * HV + h * a.V + d] = conv_silu_at(a, tail, C, row0, i, 2 * GD + h * a.V + d);
+    } else if (unit < 2 * a.G + 2 * a.H) {              // a head's decays
+        const int h = unit - 2 * a.G - a.H;
+        const float rate = expf(a.a_log[h]);
+        for (int d = lane; d < a.D; d += 64) {
+            const int c = h * a.D + d;
+            a.decay[(size_t)t * HD + c] = expf(-rate * softplus_f(a.step_pre[(size_t)t * a.step_ld + c] + a.dt_bias[c]));
+        }
+    } else {
+        for (int c = lane; c < a.H; c += 64) a.beta[(size_t)t * a.H + c] = sigmoid_ls(a.pre[(size_t)t * a.ld + a.beta_col + c]);
     }
-    for (int c = tid; c < HV; c += 256) a.v[(size_t)t * HV + c] = chan[2 * GD + c];
-    for (int c = tid; c < HD; c += 256) {
-        const float sp = softplus_f(a.step_pre[(size_t)t * HD + c] + a.dt_bias[c]);
-        a.decay[(size_t)t * HD + c] = expf(-expf(a.a_log[c / a.D]) * sp);
-    }
-    for (int c = tid; c < a.H; c += 256) a.beta[(size_t)t * a.H + c] = sigmoid_ls(a.pre[(size_t)t * a.ld + a.beta_col + c]);
 }
 
-extern "C" int llmx_delta_prep(const float* pre, int ld, const float* conv_w, const float* step_pre, const float* dt_bias, const float* a_log,
-                               const float* state, long state_stride, int tail_off, const int* slot_read, const int* row_entry,
-                               const int* entry_rows, float* q, float* k, float* v, float* decay, float* beta, int rows, int G, int H, int D, int V,
-                               int taps, int beta_col, hipStream_t stream) {
+extern "C" int llmx_delta_prep(const float* pre, int ld, const float* conv_w, const float* step_pre, int step_ld, const float* dt_bias,
+                               const float* a_log, const float* state, long state_stride, int tail_off, const int* slot_read,
+                               const int* row_entry, const int* entry_rows, float* q, float* k, float* v, float* decay, float* beta, int rows, int G,
+                               int H, int D, int V, int taps, int beta_col, hipStream_t stream) {
     if (rows <= 0) return 0;
     const long C = 2L * G * D + (long)H * V;
-    if (taps < 1 || G < 1 || H % G || C * (long)sizeof(float) > 64 * 1024 || beta_col + H > ld || C > ld) return -2;
-    DeltaPrepArgs a{pre, ld, conv_w, step_pre, dt_bias, a_log, state, state_stride, tail_off, slot_read, row_entry, entry_rows,
+    if (taps < 1 || G < 1 || H % G || D > PREP_MAX || beta_col + H > ld || C > ld || step_ld < H * D) return -2;
+    DeltaPrepArgs a{pre, ld, conv_w, step_pre, step_ld, dt_bias, a_log, state, state_stride, tail_off, slot_read, row_entry, entry_rows,
                     q, k, v, decay, beta, G, H, D, V, taps, beta_col};
     llmx_note_launch(LK_DELTA_PREP);
-    hipLaunchKernelGGL(delta_prep_kernel, dim3(rows), dim3(256), (size_t)C * sizeof(float), stream, a);
+    hipLaunchKernelGGL(delta_prep_kernel, dim3(rows, 2 * G + 2 * H + 1), dim3(64), 0, stream, a);
     return LLMX_CHECK_LAUNCH();
 }
 

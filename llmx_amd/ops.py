@@ -81,7 +81,8 @@ def _declare(h) -> None:
         "llmx_cast_rows": [P, P, I, L, P],
         "llmx_combine_rows": [P, P, F, P, P, F, I, I, I, P],
         "llmx_scale_softcap": [P, F, F, L, P],
-        "llmx_delta_prep": [P, I, P, P, P, P, P, L, I, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, P],
+        "llmx_delta_prep": [P, I, P, P, I, P, P, P, L, I, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, P],
+        "llmx_cast_cols": [P, I, P, I, I, I, P],
         "llmx_sigmoid_root": [P, P, F, P, I, I, P],
         "llmx_state_scan": [P, I, P, I, P, I, P, I, P, P, L, P, P, P, P, F, I, I, I, I, I, P, I, I, I, I, P],
         "llmx_head_norm_gate": [P, P, P, I, P, I, F, I, I, I, I, P],
@@ -502,6 +503,13 @@ def cast_rows(x: torch.Tensor, out: torch.Tensor) -> None:
     _check(lib().llmx_cast_rows(_dev(x, "x", torch.float32), _dev(out, "out"), _code(out.dtype), x.numel(), _stream()), "cast_rows")
 
 
+def cast_cols(x: torch.Tensor, out: torch.Tensor) -> None:
+    """out = x in out's type, x a float32 view [T, n] whose rows may be columns of a wider tensor."""
+    rows, n = out.shape
+    at, ld = _rows_view(x, "x", rows, n)
+    _check(lib().llmx_cast_cols(at, ld, _dev(out, "out"), _code(out.dtype), rows, n, _stream()), "cast_cols")
+
+
 def combine_rows(out: torch.Tensor, a: torch.Tensor, scale_a: float = 1.0, bias_a: Optional[torch.Tensor] = None,
                  b: Optional[torch.Tensor] = None, scale_b: float = 1.0, accumulate: bool = False) -> None:
     """out (= or +=) scale_a * (a + bias_a) + scale_b * b over float32 rows [T, n]; bias_a [n] and b may be None."""
@@ -537,8 +545,9 @@ def delta_prep(pre: torch.Tensor, conv_w: torch.Tensor, step_pre: torch.Tensor, 
     n_e = entry_rows.shape[0]
     if state.dim() != 2 or tail_off + (taps - 1) * C > state.shape[1]:
         raise KernelError("delta_prep: the state does not hold the convolution's tail")
+    step_at, step_ld = _rows_view(step_pre, "step_pre", T, H * D)
     _check(lib().llmx_delta_prep(_dev(pre, "pre", torch.float32), ld, _dev(conv_w, "conv_w", torch.float32, (C, taps)),
-                                 _dev(step_pre, "step_pre", torch.float32, (T, H * D)), _dev(dt_bias, "dt_bias", torch.float32, (H * D,)),
+                                 step_at, step_ld, _dev(dt_bias, "dt_bias", torch.float32, (H * D,)),
                                  _dev(a_log, "a_log", torch.float32, (H,)), _dev(state, "state", torch.float32), state.shape[1], int(tail_off),
                                  _dev(slot_read, "slot_read", torch.int32, (n_e,)), _dev(row_entry, "row_entry", torch.int32, (T,)),
                                  _dev(entry_rows, "entry_rows", torch.int32, (n_e, 2)), _dev(q, "q", torch.float32, (T, G * D)),
@@ -593,18 +602,6 @@ def head_norm_gate(o: torch.Tensor, weight: torch.Tensor, gate_pre: torch.Tensor
     za, ldz = _rows_view(gate_pre, "gate_pre", T, H * V)
     _check(lib().llmx_head_norm_gate(_dev(o, "o", torch.float32, (T, H * V)), _dev(weight, "weight", torch.float32, (V,)), za, ldz,
                                      _dev(out, "out", shape=(T, H * V)), _code(out.dtype), float(eps), T, H, V, int(gate), _stream()), "head_norm_gate")
-
-
-def gemm_rows_view(a: torch.Tensor, w: torch.Tensor, c: torch.Tensor) -> None:
-    """c = a @ w^T for a float32 `a` whose rows may be columns of a wider tensor (a low-rank projection's inner values,
-    left in float32): the universal product with its own row stride."""
-    M, K = a.shape
-    N = w.shape[0]
-    if w.shape[1] != K or tuple(c.shape) != (M, N) or a.stride(1) != 1 or not a.is_cuda:
-        raise KernelError("gemm_rows_view: shapes do not agree")
-    lda = a.stride(0) if M > 1 else max(K, a.stride(0))
-    _check(lib().llmx_gemm_generic(a.data_ptr(), _code(a.dtype), _dev(w, "w"), _code(w.dtype), _dev(c, "c"), _code(c.dtype),
-                                   M, N, K, lda, K, N, EPI_STORE, 0, 0, 0, 1, 0, 0, 0, 0, _stream()), "gemm")
 
 
 SKINNY_MAX_ROWS = 64          # dense products of at most this many rows stream the weights once on the matrix cores

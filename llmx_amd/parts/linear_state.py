@@ -62,8 +62,11 @@ class GatedLinearAttention(Mixer):
         pre = step.buf("gla.pre", (T, self.in_width), torch.float32)
         ops.gemm(h, self.w_in, pre, scratch=step.buf)
         view = lambda n: pre[:, self.cols[n][0]:self.cols[n][0] + self.cols[n][1]]
+        # the low-rank projection's inner values as rows of their own, in the type products read
+        inner = step.buf("gla.inner", (T, self.rank), step.act_dtype)
+        ops.cast_cols(view("a1"), inner)
         z = step.buf("gla.z", (T, H * D), torch.float32)
-        ops.gemm_rows_view(view("a1"), self.w_a2, z)
+        ops.gemm(inner, self.w_a2, z, scratch=step.buf)
         decay = step.buf("gla.decay", (T, H * D), torch.float32)
         ops.sigmoid_root(z, self.b_a2, self.tau, decay)
         o = step.buf("gla.o", (T, H * V), torch.float32)
@@ -94,14 +97,12 @@ class ChannelDeltaRule(Mixer):
             raise ValueError("delta rule: the head count must be divisible by the q/k head count")
         GD, HV, H = self.kv_heads * self.dim, self.heads * self.vdim, self.heads
         self.channels = 2 * GD + HV
-        if self.channels * 4 > 64 * 1024:
-            raise ValueError(f"delta rule: {self.channels} convolved channels a row; the preparation kernel keeps at most {64 * 1024 // 4}")
         # the fused in-projection's columns: q | k | v (the convolved channels, in this order) | b | a1 | g1
         self.cols = {"q": (0, GD), "k": (GD, GD), "v": (2 * GD, HV), "b": (self.channels, H), "a1": (self.channels + H, self.decay_rank),
                      "g1": (self.channels + H + self.decay_rank, self.gate_rank)}
         self.in_width = self.channels + H + self.decay_rank + self.gate_rank
         self.state_matrix = H * self.dim * self.vdim
-        self.w_in = self.conv = self.a_log = self.dt_bias = self.w_a2 = self.w_g2 = self.norm = self.w_o = None
+        self.w_in = self.conv = self.a_log = self.dt_bias = self.w_low = self.norm = self.w_o = None
 
     def cache_need(self):
         return StateNeed((self.state_matrix + (self.taps - 1) * self.channels,), "float32")
@@ -124,7 +125,11 @@ class ChannelDeltaRule(Mixer):
     def load(self, tensors):
         self.w_in, self.conv = tensors[self.name("in")], tensors[self.name("conv")]
         self.a_log, self.dt_bias = tensors[self.name("A_log")], tensors[self.name("dt_bias")]
-        self.w_a2, self.w_g2 = tensors[self.name("a2")], tensors[self.name("g2")]
+        # the two low-rank projections' second halves as one product: [step | gate] = [a1 h | g1 h] @ blockdiag(a2, g2)^T
+        a2, g2 = tensors[self.name("a2")], tensors[self.name("g2")]
+        self.w_low = torch.zeros((a2.shape[0] + g2.shape[0], self.decay_rank + self.gate_rank), dtype=a2.dtype, device=a2.device)
+        self.w_low[:a2.shape[0], :self.decay_rank].copy_(a2)
+        self.w_low[a2.shape[0]:, self.decay_rank:].copy_(g2)
         self.norm, self.w_o = tensors[self.name("norm")], tensors[self.name("o")]
 
     def forward(self, step, h, out, accumulate, cache: LayerCache, h32=None):
@@ -133,10 +138,13 @@ class ChannelDeltaRule(Mixer):
         pre = step.buf("delta.pre", (T, self.in_width), f32)
         ops.gemm(h, self.w_in, pre, scratch=step.buf)
         view = lambda n: pre[:, self.cols[n][0]:self.cols[n][0] + self.cols[n][1]]
-        step_pre = step.buf("delta.step", (T, H * D), f32)
-        ops.gemm_rows_view(view("a1"), self.w_a2, step_pre)
-        gate_pre = step.buf("delta.gate", (T, H * V), f32)
-        ops.gemm_rows_view(view("g1"), self.w_g2, gate_pre)
+        # both low-rank projections' inner values (neighbouring columns) as rows of their own, in the type products read
+        ranks = self.decay_rank + self.gate_rank
+        inner = step.buf("delta.inner", (T, ranks), step.act_dtype)
+        ops.cast_cols(pre[:, self.cols["a1"][0]:self.cols["a1"][0] + ranks], inner)
+        low = step.buf("delta.low", (T, H * D + H * V), f32)
+        ops.gemm(inner, self.w_low, low, scratch=step.buf)
+        step_pre, gate_pre = low[:, :H * D], low[:, H * D:]
         q, k = step.buf("delta.q", (T, G * D), f32), step.buf("delta.k", (T, G * D), f32)
         v, decay, beta = step.buf("delta.v", (T, H * V), f32), step.buf("delta.decay", (T, H * D), f32), step.buf("delta.beta", (T, H), f32)
         ops.delta_prep(pre, self.conv, step_pre, self.dt_bias, self.a_log, cache.state, self.state_matrix, step.entry_held_slots,
