@@ -1,5 +1,6 @@
 // Mixers that carry a matrix state from token to token: for every head a float32 matrix S [D key channels, V value
-// channels] in the request's state slot, updated once a token:
+// channels] in the request's state slot (stored in tiles of 8 value channels, [head][tile][D][8], the last tile padded, so
+// that the block that owns a tile reads and writes one run of memory), updated once a token:
 //     S <- diag(g_t) S                         (a decay a key channel, acting on S's rows)
 //     u  = beta_t (v_t - S^T k_t)              (delta rule; without it u = v_t: gated linear attention)
 //     S <- S + k_t u^T,   o_t = S^T q_t        (the read-out sees the token's own write)
@@ -179,7 +180,7 @@ __global__ void __launch_bounds__(128) state_scan_kernel(StateScanArgs a) {
     const int row0 = a.entry_rows[2 * e], n = a.entry_rows[2 * e + 1];
     const int j = tile * SCAN_COLS + c;
     const bool col = j < a.V;
-    const int d0 = s * R;
+    const int d0 = s * R;           // where the lane's operands lie in a staged row; its i-th key channel is 16 i + s
     const size_t slot_r = (size_t)a.slot_read[e] * a.state_stride, slot_w = (size_t)a.slot_write[e] * a.state_stride;
 
     if (a.taps > 1 && blockIdx.x == 0) {
@@ -216,22 +217,28 @@ __global__ void __launch_bounds__(128) state_scan_kernel(StateScanArgs a) {
         }
         if (a.beta) bstage = a.beta[(size_t)(row0 + min(t0 + min(tid, CH - 1), n - 1)) * a.H + h];
     };
+    // a staged row holds channel d at (d % 16) * R + d / 16, so that a lane's R values (channels s, 16 + s, ...) lie together
     auto put = [&](int b) {
 #pragma unroll
-        for (int u = 0; u < STAGE; ++u)
-            if (tid + 128 * u < CH * PER_TOKEN) (&rows[b][0][0])[tid + 128 * u] = stage[u];
+        for (int u = 0; u < STAGE; ++u) {
+            const int idx = tid + 128 * u;
+            const int tt = idx / PER_TOKEN, rem = idx % PER_TOKEN, which = rem / DP, d = rem % DP;
+            if (idx < CH * PER_TOKEN) rows[b][tt][which * DP + (d % 16) * R + d / 16] = stage[u];
+        }
         if (tid < CH * SCAN_COLS) (&vals[b][0][0])[tid] = vstage;
         if (tid < CH) betas[b][tid] = bstage;
     };
 
     fetch(0);
     float S[R];
+    const size_t tile_at = ((size_t)h * tiles + tile) * a.D * SCAN_COLS + c;
     {
-        const float* src = a.state + slot_r + ((size_t)h * a.D) * a.V + (col ? j : 0);
+        const float* src = a.state + slot_r + tile_at;
 #pragma unroll
         for (int i = 0; i < R; ++i) {
-            const float x = src[(size_t)(d0 + i < a.D ? d0 + i : 0) * a.V];
-            S[i] = (col && d0 + i < a.D) ? x : 0.0f;
+            const int d = 16 * i + s;
+            const float x = src[(size_t)(d < a.D ? d : 0) * SCAN_COLS];
+            S[i] = (col && d < a.D) ? x : 0.0f;
         }
     }
     put(0);
@@ -250,7 +257,10 @@ __global__ void __launch_bounds__(128) state_scan_kernel(StateScanArgs a) {
         nb = betas[b][tt];
     };
     for (int t0 = 0, b = 0; t0 < n; t0 += CH, b ^= 1) {
-        fetch(t0 + CH);             // past the end the last row is asked for again and never used
+        // long chunks ask for the next one whatever it is (past the end the last row again, never used): a load behind a
+        // branch would be waited for at once; steps of single tokens (CH 2) save the trip
+        const bool more = CH > 2 || t0 + CH < n;
+        if (more) fetch(t0 + CH);
         const int m = min(CH, n - t0);
         read(b, 0);
         for (int tt = 0; tt < m; ++tt) {
@@ -290,21 +300,21 @@ __global__ void __launch_bounds__(128) state_scan_kernel(StateScanArgs a) {
             const float sum = row16_sum(NC == 4 ? (o[0] + o[1]) + (o[2] + o[3]) : NC == 2 ? o[0] + o[1] : o[0]);
             if (s == 0 && col) a.out[(size_t)(row0 + t0 + tt) * a.H * a.V + (size_t)h * a.V + j] = sum * a.out_scale;
         }
-        put(b ^ 1);
+        if (more) put(b ^ 1);
         __syncthreads();
     }
     {
-        float* dst = a.state + slot_w + ((size_t)h * a.D) * a.V + j;
+        float* dst = a.state + slot_w + tile_at;
 #pragma unroll
         for (int i = 0; i < R; ++i)
-            if (col && d0 + i < a.D) dst[(size_t)(d0 + i) * a.V] = S[i];
+            if (col && 16 * i + s < a.D) dst[(size_t)(16 * i + s) * SCAN_COLS] = S[i];
     }
 }
 
 extern "C" int llmx_state_scan(const float* q, int ldq, const float* k, int ldk, const float* v, int ldv, const float* decay, int ldg,
                                const float* beta, float* state, long state_stride, const int* slot_read, const int* slot_write,
                                const int* entry_rows, float* out, float out_scale, int n_entries, int H, int share, int D, int V,
-                               const float* tail_src, int tail_ld, int tail_C, int taps, int tail_off, hipStream_t stream) {
+                               const float* tail_src, int tail_ld, int tail_C, int taps, int tail_off, int max_rows, hipStream_t stream) {
     if (n_entries <= 0) return 0;
     if (H < 1 || share < 1 || H % share || D < 1 || D > 256 || V < 1 || (taps > 1 && !tail_src)) return -2;
     StateScanArgs a{q, k, v, decay, beta, ldq, ldk, ldv, ldg, state, state_stride, slot_read, slot_write, entry_rows, out, out_scale,
@@ -312,11 +322,19 @@ extern "C" int llmx_state_scan(const float* q, int ldq, const float* k, int ldk,
     const dim3 grid((unsigned)(H * ((V + SCAN_COLS - 1) / SCAN_COLS)), (unsigned)n_entries);
     llmx_note_launch(LK_STATE_SCAN);
     const int per_lane = (D + 15) / 16;
-    if (per_lane <= 1) hipLaunchKernelGGL((state_scan_kernel<1, 8>), grid, dim3(128), 0, stream, a);
-    else if (per_lane <= 2) hipLaunchKernelGGL((state_scan_kernel<2, 8>), grid, dim3(128), 0, stream, a);
-    else if (per_lane <= 4) hipLaunchKernelGGL((state_scan_kernel<4, 8>), grid, dim3(128), 0, stream, a);
-    else if (per_lane <= 8) hipLaunchKernelGGL((state_scan_kernel<8, 8>), grid, dim3(128), 0, stream, a);
-    else hipLaunchKernelGGL((state_scan_kernel<16, 8>), grid, dim3(128), 0, stream, a);
+    // steps of single decoded tokens stage chunks of two rows (a quarter of the LDS, so more blocks a compute unit); a
+    // row's arithmetic does not depend on the chunk it came in
+#define LLMX_SCAN(R_) \
+    do { \
+        if (max_rows > 0 && max_rows <= 2) hipLaunchKernelGGL((state_scan_kernel<R_, 2>), grid, dim3(128), 0, stream, a); \
+        else hipLaunchKernelGGL((state_scan_kernel<R_, 8>), grid, dim3(128), 0, stream, a); \
+    } while (0)
+    if (per_lane <= 1) LLMX_SCAN(1);
+    else if (per_lane <= 2) LLMX_SCAN(2);
+    else if (per_lane <= 4) LLMX_SCAN(4);
+    else if (per_lane <= 8) LLMX_SCAN(8);
+    else LLMX_SCAN(16);
+#undef LLMX_SCAN
     return LLMX_CHECK_LAUNCH();
 }
 

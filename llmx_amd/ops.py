@@ -84,7 +84,7 @@ def _declare(h) -> None:
         "llmx_delta_prep": [P, I, P, P, I, P, P, P, L, I, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, P],
         "llmx_cast_cols": [P, I, P, I, I, I, P],
         "llmx_sigmoid_root": [P, P, F, P, I, I, P],
-        "llmx_state_scan": [P, I, P, I, P, I, P, I, P, P, L, P, P, P, P, F, I, I, I, I, I, P, I, I, I, I, P],
+        "llmx_state_scan": [P, I, P, I, P, I, P, I, P, P, L, P, P, P, P, F, I, I, I, I, I, P, I, I, I, I, I, P],
         "llmx_head_norm_gate": [P, P, P, I, P, I, F, I, I, I, I, P],
         "llmx_paged_attention_mfma": [P, P, P, P, P, P, P, I, I, I, P, I, P, P, P, F, I, I, I, I, I, I, I, P],
         "llmx_route_topk": [P, P, I, L, P, P, P, I, I, I, I, I, F, P, P],
@@ -563,17 +563,43 @@ def sigmoid_root(z: torch.Tensor, bias: Optional[torch.Tensor], tau: float, out:
                                    _dev(out, "out", torch.float32, (rows, n)), rows, n, _stream()), "sigmoid_root")
 
 
+STATE_TILE = 8      # value channels of a tile of a matrix state (the scan kernel's SCAN_COLS)
+
+
+def state_matrix_size(H: int, D: int, V: int) -> int:
+    """Floats a matrix state of H heads [D, V] takes in a state slot (its value channels padded to whole tiles)."""
+    return H * -(-V // STATE_TILE) * D * STATE_TILE
+
+
+def state_matrix_tiled(S: torch.Tensor) -> torch.Tensor:
+    """A state [..., H, D, V] as the scan keeps it: [..., H * tiles * D * 8], value channel j of key channel d at tile j // 8,
+    place d * 8 + j % 8 (zeros in the last tile's padding).  `state_matrix_plain` is its inverse."""
+    *lead, H, D, V = S.shape
+    tiles = -(-V // STATE_TILE)
+    padded = torch.zeros(*lead, H, D, tiles * STATE_TILE, dtype=S.dtype, device=S.device)
+    padded[..., :V] = S
+    return padded.reshape(*lead, H, D, tiles, STATE_TILE).transpose(-3, -2).reshape(*lead, H * tiles * D * STATE_TILE)
+
+
+def state_matrix_plain(flat: torch.Tensor, H: int, D: int, V: int) -> torch.Tensor:
+    tiles = -(-V // STATE_TILE)
+    lead = flat.shape[:-1]
+    return flat[..., :H * tiles * D * STATE_TILE].reshape(*lead, H, tiles, D, STATE_TILE).transpose(-3, -2).reshape(*lead, H, D, tiles * STATE_TILE)[..., :V]
+
+
 def state_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay: torch.Tensor, beta: Optional[torch.Tensor], state: torch.Tensor,
                slot_read: torch.Tensor, slot_write: torch.Tensor, entry_rows: torch.Tensor, out: torch.Tensor, out_scale: float,
-               H: int, qk_heads: int, D: int, V: int, tail=None) -> None:
+               H: int, qk_heads: int, D: int, V: int, tail=None, max_rows: int = 0) -> None:
     """The matrix-state recurrence over each entry's rows (csrc/linear_state.hip): per head S <- diag(decay) S;
     u = beta (v - S^T k) (u = v without beta); S <- S + k u^T; out = out_scale * S^T q.  q, k [T, qk_heads*D], v [T, H*V],
-    decay [T, H*D] are float32 views whose rows may be columns of wider tensors; state [slots, width] float32 holds S
-    [H, D, V] at its start, read at slot_read[e], written at slot_write[e].  `tail` = (source [T, C] view, taps, offset):
+    decay [T, H*D] are float32 views whose rows may be columns of wider tensors; state [slots, width] float32 holds S at
+    its start in tiles of 8 value channels ([H, ceil(V / 8), D, 8]: `state_matrix_size`, `state_matrix_tiled`), read at
+    slot_read[e], written at slot_write[e].  `max_rows`: the most rows an entry has, when the caller knows it (steps of
+    single tokens stage smaller chunks; the results are the same).  `tail` = (source [T, C] view, taps, offset):
     the convolution tail [taps - 1, C] at `offset` of the state is handed on from the step's rows of `source`."""
     T = out.shape[0]
     n_e = entry_rows.shape[0]
-    if H % qk_heads or state.dim() != 2 or state.shape[1] < H * D * V or D > 256:
+    if H % qk_heads or state.dim() != 2 or state.shape[1] < state_matrix_size(H, D, V) or D > 256:
         raise KernelError("state_scan: heads, widths or state do not fit")
     qa, ldq = _rows_view(q, "q", T, qk_heads * D)
     ka, ldk = _rows_view(k, "k", T, qk_heads * D)
@@ -584,12 +610,12 @@ def state_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay: torch.T
         src, taps, toff = tail
         tC = src.shape[1]
         ta, tld = _rows_view(src, "tail source", T, tC)
-        if toff < H * D * V or toff + (taps - 1) * tC > state.shape[1]:
+        if toff < state_matrix_size(H, D, V) or toff + (taps - 1) * tC > state.shape[1]:
             raise KernelError("state_scan: the state does not hold the convolution's tail")
     _check(lib().llmx_state_scan(qa, ldq, ka, ldk, va, ldv, ga, ldg, _dev(beta, "beta", torch.float32, (T, H)), _dev(state, "state", torch.float32),
                                  state.shape[1], _dev(slot_read, "slot_read", torch.int32, (n_e,)), _dev(slot_write, "slot_write", torch.int32, (n_e,)),
                                  _dev(entry_rows, "entry_rows", torch.int32, (n_e, 2)), _dev(out, "out", torch.float32, (T, H * V)), float(out_scale),
-                                 n_e, H, H // qk_heads, D, V, ta, tld, tC, int(taps), int(toff), _stream()), "state_scan")
+                                 n_e, H, H // qk_heads, D, V, ta, tld, tC, int(taps), int(toff), int(max_rows), _stream()), "state_scan")
 
 
 GATE_SIGMOID, GATE_SILU = 0, 1

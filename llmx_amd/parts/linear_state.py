@@ -7,7 +7,8 @@ Both decay S's rows channel by channel and add an outer product a token; they di
 with z_t and step_t low-rank projections of the input.  The delta rule's q, k and v first pass a short causal convolution
 over time and silu, and q and k are made unit vectors a head.  The read-out is RMS-normed a head, gated, and projected.
 Products may read rounded rows; decays, gates, unit norms, the recurrence and the state are float32 in both paths.
-The state lives in the request's slot: S [H, D, V], then (delta rule) the convolution's last taps - 1 inputs [taps - 1, C].
+The state lives in the request's slot: S (in the scan kernel's tiles of value channels), then (delta rule) the convolution's
+last taps - 1 inputs [taps - 1, C].
 """
 
 from __future__ import annotations
@@ -41,7 +42,7 @@ class GatedLinearAttention(Mixer):
         self.w_in = self.w_a2 = self.b_a2 = self.w_o = self.norm = None
 
     def cache_need(self):
-        return StateNeed((self.heads * self.dim * self.vdim,), "float32")
+        return StateNeed((ops.state_matrix_size(self.heads, self.dim, self.vdim),), "float32")
 
     def tensor_specs(self, available):
         E = self.hidden
@@ -71,7 +72,7 @@ class GatedLinearAttention(Mixer):
         ops.sigmoid_root(z, self.b_a2, self.tau, decay)
         o = step.buf("gla.o", (T, H * V), torch.float32)
         ops.state_scan(view("q"), view("k"), view("v"), decay, None, cache.state, step.entry_held_slots, step.entry_slots, step.entry_rows, o,
-                       float(D) ** -0.5, H, H, D, V)
+                       float(D) ** -0.5, H, H, D, V, max_rows=step.max_rows_per_entry)
         gated = step.buf("gla.gated", (T, H * V), step.act_dtype)
         ops.head_norm_gate(o, self.norm, view("g"), gated, self.eps, H, V, ops.GATE_SILU)
         ops.gemm(gated, self.w_o, out, ops.EPI_ADD if accumulate else ops.EPI_STORE, scratch=step.buf)
@@ -101,7 +102,7 @@ class ChannelDeltaRule(Mixer):
         self.cols = {"q": (0, GD), "k": (GD, GD), "v": (2 * GD, HV), "b": (self.channels, H), "a1": (self.channels + H, self.decay_rank),
                      "g1": (self.channels + H + self.decay_rank, self.gate_rank)}
         self.in_width = self.channels + H + self.decay_rank + self.gate_rank
-        self.state_matrix = H * self.dim * self.vdim
+        self.state_matrix = ops.state_matrix_size(H, self.dim, self.vdim)
         self.w_in = self.conv = self.a_log = self.dt_bias = self.w_low = self.norm = self.w_o = None
 
     def cache_need(self):
@@ -152,7 +153,7 @@ class ChannelDeltaRule(Mixer):
         o = step.buf("delta.o", (T, H * V), f32)
         tail = (pre[:, :self.channels], self.taps, self.state_matrix) if self.taps > 1 else None
         ops.state_scan(q, k, v, decay, beta, cache.state, step.entry_held_slots, step.entry_slots, step.entry_rows, o, float(D) ** -0.5,
-                       H, G, D, V, tail=tail)
+                       H, G, D, V, tail=tail, max_rows=step.max_rows_per_entry)
         gated = step.buf("delta.gated", (T, H * V), step.act_dtype)
         ops.head_norm_gate(o, self.norm, gate_pre, gated, self.eps, H, V, ops.GATE_SIGMOID)
         ops.gemm(gated, self.w_o, out, ops.EPI_ADD if accumulate else ops.EPI_STORE, scratch=step.buf)

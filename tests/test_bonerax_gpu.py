@@ -91,7 +91,7 @@ def test_join_of_two_results_and_logit_cap():
     assert torch.equal(z2, torch.full((2, 4), 3.0, device="cuda"))
 
 
-def _delta_case(seed, H, G, D, V, taps, entries, slots_read, slots_write, n_slots=6):
+def _delta_case(seed, H, G, D, V, taps, entries, slots_read, slots_write, n_slots=6, max_rows=0):
     """Runs delta_prep + state_scan + head_norm_gate over a step whose entries have `entries` rows each, from random
     states; returns everything the plain functions need and what the kernels gave."""
     rng = np.random.default_rng(seed)
@@ -102,20 +102,21 @@ def _delta_case(seed, H, G, D, V, taps, entries, slots_read, slots_write, n_slot
     pre = rng.normal(size=(T, ld))
     conv = rng.normal(size=(C, taps)) * 0.6
     step_pre, dt_bias, a_log = rng.normal(size=(T, H * D)), rng.normal(size=H * D), rng.normal(size=H) * 0.5 - 1.0
-    width = H * D * V + (taps - 1) * C
-    state = rng.normal(size=(n_slots, width)) * 0.5
-    state_d = dev(state)
+    matrix = o.state_matrix_size(H, D, V)       # the kernel keeps S in tiles of value channels
+    state = rng.normal(size=(n_slots, H * D * V + (taps - 1) * C)) * 0.5
+    state_d = torch.cat([o.state_matrix_tiled(dev(state[:, :H * D * V]).reshape(n_slots, H, D, V)), dev(state[:, H * D * V:])], dim=1).contiguous()
+    before = state_d.clone()
     row_entry = np.repeat(np.arange(len(entries)), entries)
     entry_rows = np.array([[sum(entries[:i]), n] for i, n in enumerate(entries)])
     q, k = torch.empty(T, G * D, device="cuda"), torch.empty(T, G * D, device="cuda")
     v, decay, beta = torch.empty(T, H * V, device="cuda"), torch.empty(T, H * D, device="cuda"), torch.empty(T, H, device="cuda")
     sr, sw = dev(slots_read, torch.int32), dev(slots_write, torch.int32)
     pre_d = dev(pre)
-    o.delta_prep(pre_d, dev(conv), dev(step_pre), dev(dt_bias), dev(a_log), state_d, H * D * V, sr, dev(row_entry, torch.int32),
+    o.delta_prep(pre_d, dev(conv), dev(step_pre), dev(dt_bias), dev(a_log), state_d, matrix, sr, dev(row_entry, torch.int32),
                  dev(entry_rows, torch.int32), q, k, v, decay, beta, G, H, D, V, C)
     out = torch.empty(T, H * V, device="cuda")
-    tail = (pre_d[:, :C], taps, H * D * V) if taps > 1 else None
-    o.state_scan(q, k, v, decay, beta, state_d, sr, sw, dev(entry_rows, torch.int32), out, D ** -0.5, H, G, D, V, tail=tail)
+    tail = (pre_d[:, :C], taps, matrix) if taps > 1 else None
+    o.state_scan(q, k, v, decay, beta, state_d, sr, sw, dev(entry_rows, torch.int32), out, D ** -0.5, H, G, D, V, tail=tail, max_rows=max_rows)
     # the plain way, entry by entry, from the slot each entry reads
     for e, n in enumerate(entries):
         r0 = entry_rows[e, 0]
@@ -141,12 +142,12 @@ def _delta_case(seed, H, G, D, V, taps, entries, slots_read, slots_write, n_slot
                 S[h] += np.outer(kk[t, h], u)
                 want[t, h] = S[h].T @ qq[t, h]
         close(out[r0:r0 + n], want.reshape(n, H * V), 2e-5, f"read-out of entry {e}")
-        got_state = state_d[slots_write[e]].cpu().double().numpy()
-        close(got_state[:H * D * V], S.reshape(-1), 2e-5, f"state of entry {e}")
+        close(o.state_matrix_plain(state_d[slots_write[e]], H, D, V), S, 2e-5, f"state of entry {e}")
         if taps > 1:
-            assert np.array_equal(got_state[H * D * V:].reshape(taps - 1, C), x[n:].astype(np.float32).astype(np.float64)), f"tail of entry {e}"
+            got_tail = state_d[slots_write[e], matrix:].cpu().double().numpy()
+            assert np.array_equal(got_tail.reshape(taps - 1, C), x[n:].astype(np.float32).astype(np.float64)), f"tail of entry {e}"
     untouched = [s for s in range(n_slots) if s not in slots_write]
-    assert torch.equal(state_d[untouched].cpu(), torch.as_tensor(state[untouched]).float())
+    assert torch.equal(state_d[untouched], before[untouched])
     return out
 
 
@@ -155,7 +156,10 @@ def test_delta_rule_rows_states_slots_and_the_convolution_tail(sizes):
     """Entries of 1, 2 (fewer than the taps: the tail is shifted), 9 and 40 rows read their state and tail at one slot and
     write them at another (and in place); slots of no entry are untouched."""
     H, G, D, V, taps = sizes
-    _delta_case(1, H, G, D, V, taps, [9, 1, 2, 40], [0, 2, 4, 5], [1, 3, 4, 0])
+    whole = _delta_case(1, H, G, D, V, taps, [9, 1, 2, 40], [0, 2, 4, 5], [1, 3, 4, 0])
+    # steps of one or two rows an entry take smaller chunks: the same bits as the rows get in the larger ones
+    short = _delta_case(2, H, G, D, V, taps, [1, 2, 1], [0, 2, 4], [1, 3, 4], max_rows=2)
+    assert torch.equal(short, _delta_case(2, H, G, D, V, taps, [1, 2, 1], [0, 2, 4], [1, 3, 4]))
 
 
 def test_matrix_state_without_the_delta_correction_and_strided_operands():
@@ -171,7 +175,7 @@ def test_matrix_state_without_the_delta_correction_and_strided_operands():
     alpha = plain.sigmoid(z + bias) ** (1.0 / 8.0)
     close(decay, alpha, 1e-6)
     state = rng.normal(size=(4, H * D * V))
-    state_d, wide_d = dev(state), dev(wide)
+    state_d, wide_d = o.state_matrix_tiled(dev(state).reshape(4, H, D, V)).contiguous(), dev(wide)
     entry_rows = np.array([[sum(entries[:i]), n] for i, n in enumerate(entries)])
     out = torch.empty(T, H * V, device="cuda")
     o.state_scan(wide_d[:, :H * D], wide_d[:, H * D:2 * H * D], wide_d[:, 2 * H * D:2 * H * D + H * V], decay, None, state_d,
@@ -183,7 +187,7 @@ def test_matrix_state_without_the_delta_correction_and_strided_operands():
         for t in range(n):
             S = S * alpha[r0 + t].reshape(H, D)[:, :, None] + k[t][:, :, None] * v[t][:, None, :]
             close(out[r0 + t], 0.25 * np.einsum("hdv,hd->hv", S, q[t]).reshape(-1), 2e-5)
-        close(state_d[[0, 2, 3][e]], S.reshape(-1), 2e-5)
+        close(o.state_matrix_plain(state_d[[0, 2, 3][e]], H, D, V), S, 2e-5)
 
 
 @pytest.mark.parametrize("gate", ["sigmoid", "silu"])
