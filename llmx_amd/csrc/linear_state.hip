@@ -129,8 +129,8 @@ extern "C" int llmx_sigmoid_root(const float* z, const float* bias, float inv_ta
 // 8 * tile + c together, lane s of them the key channels [s R, s R + R) of its head.  q and k are read head h / share (several heads may share one), with row
 // strides of their own, so they may be columns of a wider projection.  A lane's sums over its R channels run in up to four
 // chains (channels i, i + 4, ...: (c0 + c1) + (c2 + c3)); sums over a column's sixteen lanes are a butterfly over the row.
-// The block of tile 0 of an entry also hands on the convolution tail: the entry's last taps - 1 inputs, from this step's
-// rows of `tail_src` and, where the step brought fewer, from the old tail.
+// An entry's blocks also hand on the convolution tail, each a share of its channels: the entry's last taps - 1 inputs, from
+// this step's rows of `tail_src` and, where the step brought fewer, from the old tail.
 struct StateScanArgs {
     const float* q;
     const float* k;
@@ -183,10 +183,12 @@ __global__ void __launch_bounds__(128) state_scan_kernel(StateScanArgs a) {
     const int d0 = s * R;           // where the lane's operands lie in a staged row; its i-th key channel is 16 i + s
     const size_t slot_r = (size_t)a.slot_read[e] * a.state_stride, slot_w = (size_t)a.slot_write[e] * a.state_stride;
 
-    if (a.taps > 1 && blockIdx.x == 0) {
+    if (a.taps > 1) {       // the entry's blocks share the tail's channels out among themselves
         const float* old = a.state + slot_r + a.tail_off;
         float* fresh = a.state + slot_w + a.tail_off;
-        for (int ch = tid; ch < a.tail_C; ch += 128) {
+        const int share = (a.tail_C + (int)gridDim.x - 1) / (int)gridDim.x;
+        const int ch_end = min(a.tail_C, ((int)blockIdx.x + 1) * share);
+        for (int ch = (int)blockIdx.x * share + tid; ch < ch_end; ch += 128) {
             for (int p = 0; p < a.taps - 1; ++p) {      // ascending: in place, a value is read before its place is written
                 const int idx = n - (a.taps - 1) + p;
                 fresh[(size_t)p * a.tail_C + ch] = idx >= 0 ? a.tail_src[(size_t)(row0 + idx) * a.tail_ld + ch] : old[(size_t)(n + p) * a.tail_C + ch];
