@@ -174,7 +174,7 @@ __global__ void __launch_bounds__(256) cast_cols_kernel(const float* __restrict_
 extern "C" int llmx_cast_cols(const float* x, int ld, void* out, int out_dtype, int rows, int n, hipStream_t stream) {
     if (rows <= 0 || n <= 0) return 0;
     if (ld < n) return -2;
-    llmx_note_launch(LK_CAST_ROWS);
+    llmx_note_launch(LK_CAST_COLS);
     const size_t total = (size_t)rows * n;
     const dim3 grid((unsigned)((total + 255) / 256));
     if (out_dtype == LLMX_F32) hipLaunchKernelGGL(cast_cols_kernel<float>, grid, dim3(256), 0, stream, x, ld, (float*)out, n, total);

@@ -66,6 +66,7 @@
     X(LAYERNORM, "layernorm")                                                                                             \
     X(LAYERNORM_ADD, "layernorm_add")                                                                                     \
     X(CAST_ROWS, "cast_rows")                                                                                             \
+    X(CAST_COLS, "cast_cols")                                                                                             \
     X(COMBINE_ROWS, "combine_rows")                                                                                       \
     X(SCALE_SOFTCAP, "scale_softcap")                                                                                     \
     X(HEAD_NORM_ROPE_KVWRITE, "head_norm_rope_kvwrite")                                                                   \

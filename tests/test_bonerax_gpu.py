@@ -453,6 +453,33 @@ def test_long_decoding_and_graph_replays(setup):
     reference_rows(name, dtype, length, seed, whole, eager)
 
 
+def test_which_kernels_a_serving_step_takes():
+    """The launch witness: at sizes the matrix cores take (configuration A), a bfloat16 step runs the design's own kernels
+    and the matrix-core attention and products, never the universal ones; a float32 engine never launches a bfloat16
+    product.  A dispatch that fell back silently fails here, not only in a benchmark."""
+    from llmx_amd.engine import StepEntry
+    o = ops()
+    tokens = tokens_for("A", 70, 2)
+    for dtype in ("bfloat16", "float32"):
+        engine = make_engine("A", dtype, graphs=False)
+        engine.add_request("r")
+        seen = {}
+        for entry in (StepEntry("r", tokens[:69], [68]), StepEntry("r", tokens[69:], [0])):       # a prompt's portion, then one token
+            o.take_launches()
+            engine.step([entry])
+            for name, count in o.take_launches().items():
+                seen[name] = seen.get(name, 0) + count
+        for name in ("state_scan", "delta_prep", "head_norm_gate", "sigmoid_root", "layernorm_add", "layernorm", "head_norm_rope_kvwrite",
+                     "combine_rows", "scale_softcap", "route_topk", "moe_combine"):
+            assert seen.get(name), f"{dtype}: no launch of {name} ({sorted(seen)})"
+        if dtype == "bfloat16":
+            assert not any(n.startswith(("gemm_generic", "attention.generic")) for n in seen), sorted(seen)
+            assert any(n.startswith("attention.") for n in seen) and any(n.startswith("gemm_skinny") or n.startswith("gemm_tile") for n in seen)
+            assert seen.get("cast_rows") == 2        # the first layer's copy of x, once a step; later layers get theirs from the joins
+        else:
+            assert not any(n.startswith(("gemm_skinny", "gemm_tile", "attention.tiles", "attention.split", "attention.direct")) for n in seen), sorted(seen)
+
+
 def test_a_failed_step_leaves_states_and_pages_as_they_were():
     from llmx_amd.cache import OutOfPages
     from llmx_amd.engine import StepEntry
