@@ -84,9 +84,19 @@ CONFIG_C = {
     ],
     "ranks": {"0": {"decay": 8}, "1": {"decay": 16, "gate": 24}, "2": {"decay": 8, "gate": 8}},
 }
-CONFIGS = {"A": CONFIG_A, "B": CONFIG_B, "C": CONFIG_C}
-PAGES = {"A": 16, "B": 4, "C": 16}
-SEEDS = {"A": 11, "B": 12, "C": 13}
+# D: recurrent layers only (no pages at all), dense feed-forwards or none, a head wider than the model.
+CONFIG_D = {
+    "architecture": "Bonerax", "vocab": 80, "width": 48, "norm": {"eps": 1e-6}, "logit_scale": 1.5, "logit_softcap": 20.0,
+    "layers": [
+        _layer("gla", {"heads": 2, "dim": 40, "vdim": 56, "tau": 2.5}, {"kind": "dense", "ff": 72}),
+        _layer("channel_delta", _delta(4, 2, 12, 20, 3), None),
+        _layer("gla", {"heads": 2, "dim": 40, "vdim": 56, "tau": 2.5}, {"kind": "dense", "ff": 72}, weights_of=0),
+    ],
+    "ranks": {"0": {"decay": 8}, "1": {"decay": 8, "gate": 8}},
+}
+CONFIGS = {"A": CONFIG_A, "B": CONFIG_B, "C": CONFIG_C, "D": CONFIG_D}
+PAGES = {"A": 16, "B": 4, "C": 16, "D": 16}
+SEEDS = {"A": 11, "B": 12, "C": 13, "D": 14}
 
 
 def write_folder(config: dict, seed: int, folder: str, edit=None) -> str:
