@@ -4,8 +4,8 @@
 //     S <- diag(g_t) S                         (a decay a key channel, acting on S's rows)
 //     u  = beta_t (v_t - S^T k_t)              (delta rule; without it u = v_t: gated linear attention)
 //     S <- S + k_t u^T,   o_t = S^T q_t        (the read-out sees the token's own write)
-// A column of S (one value channel) never meets another, so the scan gives every column to sixteen lanes that hold a
-// sixteenth of its D values each in registers and walk a request's rows in order: the state after a row is the same bits however
+// A column of S (one value channel) never meets another, so the scan gives every column to 32 lanes that hold a
+// thirty-second of its D values each in registers and walk a request's rows in order: the state after a row is the same bits however
 // the rows were cut into steps.  Decays, gates, unit norms and the state are float32 in both number formats.
 // Around it: the preparation of a delta-rule row (short causal convolutions with silu, unit-norm q and k, the decay and
 // beta), the decay of gated linear attention, and the gated RMS norm of the read-out.
@@ -125,10 +125,11 @@ extern "C" int llmx_sigmoid_root(const float* z, const float* bias, float inv_ta
 }
 
 // ---------------------------------------------------------------------------
-// The scan.  Grid (H * ceil(V / 8), entries), two waves a block: the 16 lanes of a row of lanes own value channel
-// 8 * tile + c together, lane s of them the key channels [s R, s R + R) of its head.  q and k are read head h / share (several heads may share one), with row
+// The scan.  Grid (H * ceil(V / 8), entries), four waves a block: 32 lanes (two rows of 16) own value channel
+// 8 * tile + c together, lane s of them the key channels s, 32 + s, ... of its head (R of them).  q and k are read head h / share (several heads may share one), with row
 // strides of their own, so they may be columns of a wider projection.  A lane's sums over its R channels run in up to four
-// chains (channels i, i + 4, ...: (c0 + c1) + (c2 + c3)); sums over a column's sixteen lanes are a butterfly over the row.
+// chains (channels i, i + 4, ...: (c0 + c1) + (c2 + c3)); sums over a column's lanes are a butterfly over each row of 16,
+// then the two rows' sums added.
 // An entry's blocks also hand on the convolution tail, each a share of its channels: the entry's last taps - 1 inputs, from
 // this step's rows of `tail_src` and, where the step brought fewer, from the old tail.
 struct StateScanArgs {
@@ -155,32 +156,28 @@ struct StateScanArgs {
 // token to token waits for LDS, not for memory; a token's operands are read from LDS while the token before is worked on.
 // Every load is asked for whatever the index (addresses are clamped, the value is chosen afterwards), so none sits behind
 // a branch.
-__device__ __forceinline__ float row16_sum(float v) {      // the sum over a row of 16 lanes, the same bits in each
-    v += row_rotate<8>(v);
-    v += row_rotate<4>(v);
-    v += row_rotate<2>(v);
-    v += row_rotate<1>(v);
-    return v;
-}
+__device__ __forceinline__ float column_sum(float v) { return wave_sum(v); }     // over a column's lanes, the same bits in each
 
-#define SCAN_COLS 8     // value channels a block of two waves owns
+#define SCAN_COLS 8     // value channels a block of four waves owns
+#define SCAN_LANES 64   // lanes that share a column: a wave
+#define SCAN_THREADS (SCAN_COLS * SCAN_LANES)
 template <int R, int CH>
-__global__ void __launch_bounds__(128) state_scan_kernel(StateScanArgs a) {
-    constexpr int DP = 16 * R;                      // a head's key channels, padded
+__global__ void __launch_bounds__(SCAN_THREADS) state_scan_kernel(StateScanArgs a) {
+    constexpr int DP = SCAN_LANES * R;              // a head's key channels, padded
     constexpr int PER_TOKEN = 3 * DP;               // k | q | decay
-    constexpr int STAGE = (CH * PER_TOKEN + 127) / 128;   // values a thread brings a chunk
+    constexpr int STAGE = (CH * PER_TOKEN + SCAN_THREADS - 1) / SCAN_THREADS;   // values a thread brings a chunk
     constexpr int NC = R >= 4 ? 4 : R;              // chains a lane's sums run in
     __shared__ __attribute__((aligned(16))) float rows[2][CH][PER_TOKEN];
     __shared__ float vals[2][CH][SCAN_COLS];
     __shared__ float betas[2][CH];
-    const int tid = threadIdx.x, lane = tid & 63, s = lane & 15, c = (tid >> 4);     // c: 0..7, the block's column
+    const int tid = threadIdx.x, s = tid & (SCAN_LANES - 1), c = tid / SCAN_LANES;     // c: 0..7, the block's column; s: the lane's place in it
     const int tiles = (a.V + SCAN_COLS - 1) / SCAN_COLS;
     const int h = blockIdx.x / tiles, tile = blockIdx.x % tiles;
     const int e = blockIdx.y;
     const int row0 = a.entry_rows[2 * e], n = a.entry_rows[2 * e + 1];
     const int j = tile * SCAN_COLS + c;
     const bool col = j < a.V;
-    const int d0 = s * R;           // where the lane's operands lie in a staged row; its i-th key channel is 16 i + s
+    const int d0 = s * R;           // where the lane's operands lie in a staged row; its i-th key channel is 32 i + s
     const size_t slot_r = (size_t)a.slot_read[e] * a.state_stride, slot_w = (size_t)a.slot_write[e] * a.state_stride;
 
     if (a.taps > 1) {       // the entry's blocks share the tail's channels out among themselves
@@ -188,7 +185,7 @@ __global__ void __launch_bounds__(128) state_scan_kernel(StateScanArgs a) {
         float* fresh = a.state + slot_w + a.tail_off;
         const int share = (a.tail_C + (int)gridDim.x - 1) / (int)gridDim.x;
         const int ch_end = min(a.tail_C, ((int)blockIdx.x + 1) * share);
-        for (int ch = (int)blockIdx.x * share + tid; ch < ch_end; ch += 128) {
+        for (int ch = (int)blockIdx.x * share + tid; ch < ch_end; ch += SCAN_THREADS) {
             for (int p = 0; p < a.taps - 1; ++p) {      // ascending: in place, a value is read before its place is written
                 const int idx = n - (a.taps - 1) + p;
                 fresh[(size_t)p * a.tail_C + ch] = idx >= 0 ? a.tail_src[(size_t)(row0 + idx) * a.tail_ld + ch] : old[(size_t)(n + p) * a.tail_C + ch];
@@ -205,7 +202,7 @@ __global__ void __launch_bounds__(128) state_scan_kernel(StateScanArgs a) {
     auto fetch = [&](int t0) {
 #pragma unroll
         for (int u = 0; u < STAGE; ++u) {
-            const int idx = min(tid + 128 * u, CH * PER_TOKEN - 1);
+            const int idx = min(tid + SCAN_THREADS * u, CH * PER_TOKEN - 1);
             const int tt = idx / PER_TOKEN, rem = idx % PER_TOKEN, which = rem / DP, d = rem % DP;
             const size_t row = (size_t)(row0 + min(t0 + tt, n - 1));
             const int dd = d < a.D ? d : 0;
@@ -213,19 +210,19 @@ __global__ void __launch_bounds__(128) state_scan_kernel(StateScanArgs a) {
             const float x = src[dd];
             stage[u] = d < a.D ? x : 0.0f;
         }
-        if (CH * SCAN_COLS <= 128 || tid < CH * SCAN_COLS) {
+        if (tid < CH * SCAN_COLS) {
             const int tt = min(tid / SCAN_COLS, CH - 1), cc = tid % SCAN_COLS;
             vstage = vp[(size_t)(row0 + min(t0 + tt, n - 1)) * a.ldv + min(cc, a.V - 1 - tile * SCAN_COLS)];
         }
         if (a.beta) bstage = a.beta[(size_t)(row0 + min(t0 + min(tid, CH - 1), n - 1)) * a.H + h];
     };
-    // a staged row holds channel d at (d % 16) * R + d / 16, so that a lane's R values (channels s, 16 + s, ...) lie together
+    // a staged row holds channel d at (d % 32) * R + d / 32, so that a lane's R values (channels s, 32 + s, ...) lie together
     auto put = [&](int b) {
 #pragma unroll
         for (int u = 0; u < STAGE; ++u) {
-            const int idx = tid + 128 * u;
+            const int idx = tid + SCAN_THREADS * u;
             const int tt = idx / PER_TOKEN, rem = idx % PER_TOKEN, which = rem / DP, d = rem % DP;
-            if (idx < CH * PER_TOKEN) rows[b][tt][which * DP + (d % 16) * R + d / 16] = stage[u];
+            if (idx < CH * PER_TOKEN) rows[b][tt][which * DP + (d % SCAN_LANES) * R + d / SCAN_LANES] = stage[u];
         }
         if (tid < CH * SCAN_COLS) (&vals[b][0][0])[tid] = vstage;
         if (tid < CH) betas[b][tid] = bstage;
@@ -238,7 +235,7 @@ __global__ void __launch_bounds__(128) state_scan_kernel(StateScanArgs a) {
         const float* src = a.state + slot_r + tile_at;
 #pragma unroll
         for (int i = 0; i < R; ++i) {
-            const int d = 16 * i + s;
+            const int d = SCAN_LANES * i + s;
             const float x = src[(size_t)(d < a.D ? d : 0) * SCAN_COLS];
             S[i] = (col && d < a.D) ? x : 0.0f;
         }
@@ -246,62 +243,77 @@ __global__ void __launch_bounds__(128) state_scan_kernel(StateScanArgs a) {
     put(0);
     __syncthreads();
     const bool delta = a.beta != nullptr;
-    float nk[R], nq[R], ng[R], nv, nb;
-    auto read = [&](int b, int tt) {
+    // a token's operands as the lane reads them from the staged chunk; two sets take turns, so that a token's are read while
+    // the token before is worked on and nothing is copied from set to set
+    struct Operands {
+        float k[R], q[R], g[R], v, beta;
+    };
+    auto read = [&](Operands& x, int b, int tt) {
         const float* kr = &rows[b][tt][d0];
 #pragma unroll
         for (int i = 0; i < R; ++i) {
-            nk[i] = kr[i];
-            nq[i] = kr[DP + i];
-            ng[i] = kr[2 * DP + i];
+            x.k[i] = kr[i];
+            x.q[i] = kr[DP + i];
+            x.g[i] = kr[2 * DP + i];
         }
-        nv = vals[b][tt][c];
-        nb = betas[b][tt];
+        x.v = vals[b][tt][c];
+        x.beta = betas[b][tt];
     };
+    const size_t out_ld = (size_t)a.H * a.V;
+    // one token: the state's update, and the lane's share of the read-out (summed over the column's lanes later, for a whole
+    // chunk at once: only the delta correction's sum lies on the way from a token's state to the next one's)
+    auto token = [&](const Operands& x) -> float {
+        float u = x.v;
+        if (delta) {
+            float p[NC];
+#pragma unroll
+            for (int y = 0; y < NC; ++y) p[y] = 0.0f;
+#pragma unroll
+            for (int i = 0; i < R; ++i) {
+                S[i] = S[i] * x.g[i];
+                p[i % NC] = fmaf(x.k[i], S[i], p[i % NC]);
+            }
+            const float dot = NC == 4 ? (p[0] + p[1]) + (p[2] + p[3]) : NC == 2 ? p[0] + p[1] : p[0];
+            u = x.beta * (u - column_sum(dot));
+        } else {
+#pragma unroll
+            for (int i = 0; i < R; ++i) S[i] = S[i] * x.g[i];
+        }
+        float o[NC];
+#pragma unroll
+        for (int y = 0; y < NC; ++y) o[y] = 0.0f;
+#pragma unroll
+        for (int i = 0; i < R; ++i) {
+            S[i] = fmaf(x.k[i], u, S[i]);
+            o[i % NC] = fmaf(x.q[i], S[i], o[i % NC]);
+        }
+        return NC == 4 ? (o[0] + o[1]) + (o[2] + o[3]) : NC == 2 ? o[0] + o[1] : o[0];
+    };
+    Operands first, second;
+    float* out_at = a.out + (size_t)row0 * out_ld + (size_t)h * a.V + (col ? j : 0);
     for (int t0 = 0, b = 0; t0 < n; t0 += CH, b ^= 1) {
         // long chunks ask for the next one whatever it is (past the end the last row again, never used): a load behind a
         // branch would be waited for at once; steps of single tokens (CH 2) save the trip
         const bool more = CH > 2 || t0 + CH < n;
         if (more) fetch(t0 + CH);
         const int m = min(CH, n - t0);
-        read(b, 0);
-        for (int tt = 0; tt < m; ++tt) {
-            float ck[R], cq[R], cg[R];
+        read(first, b, 0);
+        float share[CH];
 #pragma unroll
-            for (int i = 0; i < R; ++i) {
-                ck[i] = nk[i];
-                cq[i] = nq[i];
-                cg[i] = ng[i];
+        for (int tt = 0; tt < CH; ++tt) {
+            if (tt < m) {
+                read((tt & 1) ? first : second, b, tt + 1 < CH ? tt + 1 : tt);
+                share[tt] = token((tt & 1) ? second : first);
             }
-            float u = nv;
-            const float cb = nb;
-            read(b, tt + 1 < CH ? tt + 1 : tt);
-            if (delta) {
-                float p[NC];
-#pragma unroll
-                for (int x = 0; x < NC; ++x) p[x] = 0.0f;
-#pragma unroll
-                for (int i = 0; i < R; ++i) {
-                    S[i] = S[i] * cg[i];
-                    p[i % NC] = fmaf(ck[i], S[i], p[i % NC]);
-                }
-                const float dot = NC == 4 ? (p[0] + p[1]) + (p[2] + p[3]) : NC == 2 ? p[0] + p[1] : p[0];
-                u = cb * (u - row16_sum(dot));
-            } else {
-#pragma unroll
-                for (int i = 0; i < R; ++i) S[i] = S[i] * cg[i];
-            }
-            float o[NC];
-#pragma unroll
-            for (int x = 0; x < NC; ++x) o[x] = 0.0f;
-#pragma unroll
-            for (int i = 0; i < R; ++i) {
-                S[i] = fmaf(ck[i], u, S[i]);
-                o[i % NC] = fmaf(cq[i], S[i], o[i % NC]);
-            }
-            const float sum = row16_sum(NC == 4 ? (o[0] + o[1]) + (o[2] + o[3]) : NC == 2 ? o[0] + o[1] : o[0]);
-            if (s == 0 && col) a.out[(size_t)(row0 + t0 + tt) * a.H * a.V + (size_t)h * a.V + j] = sum * a.out_scale;
         }
+#pragma unroll
+        for (int tt = 0; tt < CH; ++tt) {
+            if (tt < m) {
+                const float sum = column_sum(share[tt]);
+                if (s == 0 && col) out_at[(size_t)tt * out_ld] = sum * a.out_scale;
+            }
+        }
+        out_at += (size_t)CH * out_ld;
         if (more) put(b ^ 1);
         __syncthreads();
     }
@@ -309,7 +321,7 @@ __global__ void __launch_bounds__(128) state_scan_kernel(StateScanArgs a) {
         float* dst = a.state + slot_w + tile_at;
 #pragma unroll
         for (int i = 0; i < R; ++i)
-            if (col && 16 * i + s < a.D) dst[(size_t)(16 * i + s) * SCAN_COLS] = S[i];
+            if (col && SCAN_LANES * i + s < a.D) dst[(size_t)(SCAN_LANES * i + s) * SCAN_COLS] = S[i];
     }
 }
 
@@ -323,19 +335,19 @@ extern "C" int llmx_state_scan(const float* q, int ldq, const float* k, int ldk,
                     H, share, D, V, tail_src, tail_ld, tail_C, taps, tail_off};
     const dim3 grid((unsigned)(H * ((V + SCAN_COLS - 1) / SCAN_COLS)), (unsigned)n_entries);
     llmx_note_launch(LK_STATE_SCAN);
-    const int per_lane = (D + 15) / 16;
+    const int per_lane = (D + SCAN_LANES - 1) / SCAN_LANES;
     // steps of single decoded tokens stage chunks of two rows (a quarter of the LDS, so more blocks a compute unit); a
     // row's arithmetic does not depend on the chunk it came in
-#define LLMX_SCAN(R_) \
+#define LLMX_SCAN(R_, CH_) \
     do { \
-        if (max_rows > 0 && max_rows <= 2) hipLaunchKernelGGL((state_scan_kernel<R_, 2>), grid, dim3(128), 0, stream, a); \
-        else hipLaunchKernelGGL((state_scan_kernel<R_, 8>), grid, dim3(128), 0, stream, a); \
+        if (max_rows > 0 && max_rows <= 2) hipLaunchKernelGGL((state_scan_kernel<R_, 2>), grid, dim3(SCAN_THREADS), 0, stream, a); \
+        else hipLaunchKernelGGL((state_scan_kernel<R_, CH_>), grid, dim3(SCAN_THREADS), 0, stream, a); \
     } while (0)
-    if (per_lane <= 1) LLMX_SCAN(1);
-    else if (per_lane <= 2) LLMX_SCAN(2);
-    else if (per_lane <= 4) LLMX_SCAN(4);
-    else if (per_lane <= 8) LLMX_SCAN(8);
-    else LLMX_SCAN(16);
+    // chunks of 16 rows where LDS holds two of them (heads of at most 128 key channels): a chunk's work then outlasts the
+    // next chunk's way from memory
+    if (per_lane <= 1) LLMX_SCAN(1, 16);
+    else if (per_lane <= 2) LLMX_SCAN(2, 16);
+    else LLMX_SCAN(4, 8);
 #undef LLMX_SCAN
     return LLMX_CHECK_LAUNCH();
 }
