@@ -23,6 +23,9 @@ from .nenotar import RotaryScaling
 from .reader import ConfigError, KeyReader
 
 ARCHITECTURE = "Bonerax"
+#: keys a model folder's config.json may carry that say nothing about the arithmetic (how the folder was made, what it is
+#: called, how its file stores numbers: the loader reads the stored type from the file itself)
+WITHOUT_EFFECT = ("name", "seed", "comment", "description", "dtype", "torch_dtype")
 LAYER_TYPES = ("gla", "channel_delta", "parallel")
 MLP_KINDS = ("dense", "moe")
 
@@ -117,7 +120,7 @@ class BoneraxConfig:
         cfg = cls(vocab=r.integer("vocab"), width=r.integer("width"), norm_eps=eps, logit_scale=r.real("logit_scale", default=1.0),
                   logit_softcap=cap, layers=layers,
                   ranks=None if ranks is None else {int(k): {str(a): int(b) for a, b in v.items()} for k, v in ranks.items()})
-        r.finish((), ARCHITECTURE)
+        r.finish(WITHOUT_EFFECT, ARCHITECTURE)
         return cfg
 
     @property
@@ -215,7 +218,7 @@ def _read_layer(entry, i: int) -> LayerConfig:
             router.finish((), ARCHITECTURE)
         mlp.finish((), ARCHITECTURE)
     weights_of = r.integer("weights_of", lo=0, default=None)
-    r.finish((), ARCHITECTURE)
+    r.finish(("name", "comment"), ARCHITECTURE)
     return LayerConfig(kind, mixer, ff, weights_of)
 
 

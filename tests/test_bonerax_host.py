@@ -144,6 +144,11 @@ def test_configuration_reads_writes_and_refuses():
     refused(lambda c: c["layers"][0]["mlp"]["router"].update(top=7), r"layers\[0\].mlp.router.top")
     refused(lambda c: c["layers"][0]["mixer"]["right"].update(kv_heads=3), r"layers\[0\].mixer.right.kv_heads")
     refused(lambda c: c["layers"][0]["mixer"]["left"]["rot"].update(dims=34), r"layers\[0\].mixer.left.rot.dims")
+    refused(lambda c: c.update(tie_embeddings=True), r"key tie_embeddings is not one this engine reads")
+    # keys that say nothing about the arithmetic are let through
+    named = copy.deepcopy(CONFIG_A)
+    named.update(name="a", seed=3, dtype="bfloat16")
+    assert read_config(named) == read_config(copy.deepcopy(CONFIG_A))
     # without the inner widths a configuration cannot be assembled; a model folder's tensor shapes give them
     from llmx_amd.models import assemble, read_model_dir
     bare = {k: v for k, v in CONFIG_A.items() if k != "ranks"}
